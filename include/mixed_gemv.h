@@ -1,0 +1,177 @@
+/*
+ * mixed_gemv.h — C-ABI of the MI355X (gfx950) weight-only-quantised GEMV library.
+ *
+ *     y[b][n] = fp16( sum_k dequant(W)[n][k] * x[b][k]  (+ bias[n]) )
+ *
+ * int4 or int8 weights, fp16 activations, fp32 accumulation, fp16 output.  The entry
+ * points below are what a binding of JJXiangJiaoJun/mixed_gemv's C++ call sites needs; each
+ * one names the reference interface it stands in for.  Dimension names follow the model
+ * view: n_out = output features (the reference's M), k = reduction length, m_batch =
+ * activation rows (the reference's N, fixed to 1 there).
+ *
+ * Conventions
+ *   - fp16 values cross the ABI as uint16_t bit patterns (IEEE-754 binary16).
+ *   - Functions taking a `stream` work on DEVICE pointers, enqueue asynchronously on that
+ *     HIP stream (NULL = the null stream), never allocate and never synchronise.
+ *   - Functions without a `stream` are host utilities working on HOST pointers.
+ *   - Every function returns an mgemv_status; none prints or calls exit().  The conditions
+ *     on which the reference prints a message and exits are reported as error codes.
+ *   - The library keeps no per-call state: calls from several host threads on different
+ *     streams are safe.
+ */
+#ifndef MIXED_GEMV_H_
+#define MIXED_GEMV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(MGEMV_BUILDING_LIBRARY)
+#define MGEMV_API __attribute__((visibility("default")))
+#else
+#define MGEMV_API
+#endif
+
+/* Status codes. */
+typedef enum mgemv_status {
+  MGEMV_OK = 0,
+  MGEMV_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+  MGEMV_ERR_RANK = 2,           /* shape rank not 2 or 3 (utils/preprocess.h:486-489) */
+  MGEMV_ERR_ROWS = 3,           /* n_out not a multiple of 4 (utils/preprocess.h:319-322) */
+  MGEMV_ERR_COLS = 4,           /* k not a multiple of the 128-bit access (utils/preprocess.h:324-327) */
+  MGEMV_ERR_GROUP_SIZE = 5,     /* group_size < 64 (gemv/device/gemv_adaptor.h:199-203), not a multiple of 32, or not dividing k */
+  MGEMV_ERR_QUANT_OP = 6,       /* quant_op not 1, 2 or 3 (gemv/weight_only_quant_op.h:12-18) */
+  MGEMV_ERR_QUANT_TYPE = 7,     /* weight type not W8_A16 / W4_A16 (utils/preprocess.h:110, 287-288) */
+  MGEMV_ERR_BATCH = 8,          /* batch_count < 1 or m_batch outside [1, MGEMV_MAX_M_BATCH] */
+  MGEMV_ERR_LAYOUT = 9,         /* layout flag not row/column major, or a row-major transpose whose dims are not multiples of 64 elements (utils/preprocess.h:157-162) */
+  MGEMV_ERR_SIZE = 10,          /* a dimension is <= 0 or overflows the 32-bit index space of the kernels */
+  MGEMV_ERR_LAUNCH = 11,        /* the HIP runtime refused the launch (gemv/device/gemv_adaptor.h:249-254) */
+  MGEMV_ERR_NO_DEVICE = 12,     /* no usable gfx950 device */
+  MGEMV_ERR_ALIGNMENT = 13      /* a device pointer is not aligned as required (16 B weights/activations, 4 B scales) */
+} mgemv_status;
+
+/* gemv/weight_only_quant_op.h:12-18 — same numeric values. */
+enum {
+  MGEMV_PER_COLUMN_SCALE_ONLY = 1,
+  MGEMV_FINEGRAINED_SCALE_ONLY = 2,
+  MGEMV_FINEGRAINED_SCALE_AND_ZEROS = 3
+};
+
+/* utils/type_base.h:7-11 — same numeric values (W4_AFP8 = 2 has no kernel in the reference and none here). */
+enum { MGEMV_W8_A16 = 0, MGEMV_W4_A16 = 1 };
+
+/* utils/type_base.h:13-16 — same numeric values. */
+enum { MGEMV_ROW_MAJOR = 0, MGEMV_COLUMN_MAJOR = 1 };
+
+#define MGEMV_MAX_M_BATCH 16
+
+/* Human-readable text for a status code (never NULL). */
+MGEMV_API const char *mgemv_status_string(int status);
+
+/* Library version, major*10000 + minor*100 + patch. */
+MGEMV_API int mgemv_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Host utilities
+ * ---------------------------------------------------------------------------------------- */
+
+/* Replaces SubBytePacker<int4b_t,int8_t>::pack (utils/preprocess.h:55-84).
+ * Packs n_unpacked (even) signed 4-bit values held one per int8 into n_unpacked/2 bytes:
+ * element 2i in bits 0..3 of byte i, element 2i+1 in bits 4..7.  Values are truncated to
+ * their low 4 bits, as in the reference. */
+MGEMV_API int mgemv_pack_int4(uint8_t *packed, const int8_t *unpacked, size_t n_unpacked);
+
+/* Replaces SubBytePacker<int4b_t,int8_t>::unpack (utils/preprocess.h:41-53): sign-extending inverse. */
+MGEMV_API int mgemv_unpack_int4(int8_t *unpacked, const uint8_t *packed, size_t n_packed);
+
+/* Replaces ZeroPointPreprocessor<half_t,int8_t>::neg_zero_point_multiplies_scale
+ * (utils/preprocess.h:94-101): out[i] = fp16(-zeros[i]) * scales[i], one fp16 multiply.
+ * The result is the additive term the GEMV takes as `zero_add` (mixed_gemv_test.cu:237-239, 275). */
+MGEMV_API int mgemv_fold_zero_points(uint16_t *out, const uint16_t *scales, const int8_t *zeros, size_t n);
+
+/* Bytes that mgemv_preprocess_weights writes for this shape (>= the input size: rows are
+ * padded to 16 and k to one wave step).  shape as in mgemv_preprocess_weights.  Returns 0
+ * for an invalid rank / quant_type. */
+MGEMV_API size_t mgemv_preprocessed_size(const size_t *shape, int rank, int quant_type);
+
+/* Replaces MixedGemvWeightPreprocessor::run (utils/preprocess.h:482-522).
+ *   src     quantised weights: int4 packed two per byte (low nibble = even element) or int8.
+ *   shape   {k, n_out} or {experts, k, n_out}, exactly the reference's `shape` argument.
+ *   layout  MGEMV_COLUMN_MAJOR: memory is n_out rows of k elements (the reference's shipped
+ *           call, mixed_gemv_test.cu:247-254); MGEMV_ROW_MAJOR: memory is k rows of n_out
+ *           elements and is transposed first (utils/preprocess.h:507-511).
+ *   quant_type MGEMV_W4_A16 or MGEMV_W8_A16 (the reference's interleave rejects W8_A16,
+ *           utils/preprocess.h:350-362; here both are laid out).
+ * Same input meaning as the reference, different OUTPUT layout: the gfx950 tile layout
+ * consumed by mgemv_gemv (16-row tiles, 1 KiB wave-contiguous blocks, biased nibbles in
+ * converter order).  dst must hold mgemv_preprocessed_size() bytes and may not alias src. */
+MGEMV_API int mgemv_preprocess_weights(uint8_t *dst, const uint8_t *src, const size_t *shape, int rank,
+                                       int layout, int quant_type);
+
+/* Inverse of mgemv_preprocess_weights for MGEMV_COLUMN_MAJOR input: recovers the n_out x k
+ * row-major quantised weights from a preprocessed buffer.  No counterpart in the reference;
+ * it exists so that layouts can be audited and round-trip tested. */
+MGEMV_API int mgemv_unpreprocess_weights(uint8_t *dst, const uint8_t *src_preprocessed, const size_t *shape,
+                                         int rank, int quant_type);
+
+/* ------------------------------------------------------------------------------------------
+ * Device entry points
+ * ---------------------------------------------------------------------------------------- */
+
+/* Replaces device_gemv (mixed_gemv_test.cu:124-165) and GemvAdaptor::initialize + run
+ * (gemv/device/gemv_adaptor.h:198-255) for batch_count == 1.
+ *   weights   preprocessed weights (device), output of mgemv_preprocess_weights
+ *   x         activations, m_batch rows of k fp16, row stride k   (reference ref_B, ldb = 0 for its single row)
+ *   scale     fp16 [k/group_size][n_out], n_out contiguous (reference ref_scale, ld = n_out);
+ *             per-column mode: [n_out]
+ *   zero_add  fp16 additive term -z*s, same shape as scale; read only in mode 3
+ *             (mixed_gemv_test.cu:145-147), may be NULL otherwise
+ *   bias      fp16 [n_out] added in fp32 before the final rounding, or NULL
+ *             (reference ref_C with a source-enabled epilogue, epilogue/threadblock/epilogue.h:50-75)
+ *   y         fp16 output, m_batch rows of n_out, row stride n_out (reference ref_D, ldd = n_out)
+ *   group_size ignored (taken as k) in per-column mode (mixed_gemv_test.cu:142-143)
+ *   quant_op  MGEMV_PER_COLUMN_SCALE_ONLY / _FINEGRAINED_SCALE_ONLY / _FINEGRAINED_SCALE_AND_ZEROS,
+ *             a run-time argument here, a template parameter in the reference
+ *   weight_bits 4 or 8
+ * Dequantisation is fp16 multiply then fp16 add, separately rounded
+ * (gemv/warp/warp_dequantizer.h:52-59), accumulation is fp32. */
+MGEMV_API int mgemv_gemv(const void *weights, const uint16_t *x, const uint16_t *scale, const uint16_t *zero_add,
+                         const uint16_t *bias, uint16_t *y, int n_out, int m_batch, int k, int group_size,
+                         int quant_op, int weight_bits, void *stream);
+
+/* As mgemv_gemv, with the reference's batch arguments (gemv/device/gemv_adaptor.h:129-135;
+ * gemv/kernel/mixed_gemv.h:140-149, 222-223): batch_count independent problems, operand
+ * pointers advanced per problem by the given strides.  stride_weights is in BYTES of the
+ * preprocessed buffer (mgemv_preprocessed_size of one matrix for expert-stacked weights);
+ * the other strides are in fp16 elements; stride_scale applies to scale and zero_add,
+ * stride_bias to bias.  A stride of 0 shares the operand between problems. */
+MGEMV_API int mgemv_gemv_batched(const void *weights, const uint16_t *x, const uint16_t *scale,
+                                 const uint16_t *zero_add, const uint16_t *bias, uint16_t *y, int batch_count,
+                                 int n_out, int m_batch, int k, int group_size, int quant_op, int weight_bits,
+                                 int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
+                                 int64_t stride_bias, int64_t stride_y, void *stream);
+
+/* Parity/debug entry: writes the dequantised weights, fp16 [n_out][k] row-major, produced by
+ * the SAME device conversion and dequantisation code the GEMV kernels use
+ * (gemv/interleaved_numeric_conversion.h:62-81, 232-291 then gemv/warp/warp_dequantizer.h:52-59, 86-92).
+ * No direct counterpart in the reference, where this value only exists in registers. */
+MGEMV_API int mgemv_dequantize(const void *weights, const uint16_t *scale, const uint16_t *zero_add,
+                               uint16_t *out, int n_out, int k, int group_size, int quant_op, int weight_bits,
+                               void *stream);
+
+/* Launch geometry override for tuning and tests: k-split waves per tile and tiles per
+ * workgroup; 0 restores the built-in heuristic.  Process-wide. */
+MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup);
+
+/* Reports the geometry mgemv_gemv would use: out[0] = workgroups, out[1] = threads per
+ * workgroup, out[2] = k-split waves per tile, out[3] = tiles per workgroup,
+ * out[4] = wave steps per wave, out[5] = 1 when the matrix-core path is chosen. */
+MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[6]);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MIXED_GEMV_H_ */

@@ -1,0 +1,24 @@
+"""MI355X-native weight-only-quantised GEMV (int4/int8 weights x fp16 activations).
+
+Python mirror of the reference's host-side interface (names and argument meaning follow
+mixed_gemv_test.cu, utils/preprocess.h and gemv/device/gemv_adaptor.h of
+JJXiangJiaoJun/mixed_gemv) on top of the C-ABI in include/mixed_gemv.h.
+"""
+from .api import (  # noqa: F401
+    GemvAdaptor,
+    LayoutType,
+    MixedGemvWeightPreprocessor,
+    QuantType,
+    SubBytePacker,
+    WeightOnlyQuantOp,
+    ZeroPointPreprocessor,
+    dequantize,
+    device_gemv,
+    preprocessed_size,
+    query_launch,
+    set_launch_override,
+    unpreprocess_weights,
+)
+from ._lib import LIB_PATH, MixedGemvError  # noqa: F401
+
+__version__ = "0.1.0"

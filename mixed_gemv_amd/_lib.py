@@ -1,0 +1,64 @@
+"""ctypes binding of libmixed_gemv_amd.so (the C-ABI declared in include/mixed_gemv.h).
+
+There is no fallback: if the HIP library has not been built, importing a device entry point
+raises.  Build it with `python -m mixed_gemv_amd.build`.
+"""
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "lib", "libmixed_gemv_amd.so")
+
+_c = ctypes
+_u16p = _c.c_void_p  # fp16 bit patterns; passed as raw addresses (host numpy or device pointers)
+_vp = _c.c_void_p
+_szp = _c.POINTER(_c.c_size_t)
+
+# name -> (restype, argtypes); must list every function include/mixed_gemv.h declares
+SIGNATURES = {
+    "mgemv_status_string": (_c.c_char_p, [_c.c_int]),
+    "mgemv_version": (_c.c_int, []),
+    "mgemv_pack_int4": (_c.c_int, [_vp, _vp, _c.c_size_t]),
+    "mgemv_unpack_int4": (_c.c_int, [_vp, _vp, _c.c_size_t]),
+    "mgemv_fold_zero_points": (_c.c_int, [_u16p, _u16p, _vp, _c.c_size_t]),
+    "mgemv_preprocessed_size": (_c.c_size_t, [_szp, _c.c_int, _c.c_int]),
+    "mgemv_preprocess_weights": (_c.c_int, [_vp, _vp, _szp, _c.c_int, _c.c_int, _c.c_int]),
+    "mgemv_unpreprocess_weights": (_c.c_int, [_vp, _vp, _szp, _c.c_int, _c.c_int]),
+    "mgemv_gemv": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 6 + [_vp]),
+    "mgemv_gemv_batched": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 7
+                           + [_c.c_int64] * 5 + [_vp]),
+    "mgemv_dequantize": (_c.c_int, [_vp, _u16p, _u16p, _u16p] + [_c.c_int] * 5 + [_vp]),
+    "mgemv_set_launch_override": (_c.c_int, [_c.c_int, _c.c_int]),
+    "mgemv_query_launch": (_c.c_int, [_c.c_int] * 4 + [_c.POINTER(_c.c_int * 6)]),
+}
+
+_lib = None
+
+
+class MixedGemvError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = int(status)
+        text = lib().mgemv_status_string(self.status).decode()
+        super().__init__(f"{where}: status {self.status} ({text})")
+
+
+def lib():
+    """Loads the shared library once; raises if it is missing."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} not found: the HIP library is not built "
+                "(run `python -m mixed_gemv_amd.build`); there is no CPU fallback")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status, where):
+    if status != 0:
+        raise MixedGemvError(status, where)

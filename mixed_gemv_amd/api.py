@@ -1,0 +1,219 @@
+"""Host-side mirror of the reference's operator interface, bound to the C-ABI.
+
+Host utilities take and return numpy arrays.  Device entry points take anything exposing a
+device address: a torch tensor on the GPU, or a plain integer address.  PyTorch is used only
+as the owner of device memory and streams.
+"""
+import ctypes
+import enum
+
+import numpy as np
+
+from . import _lib
+
+
+class WeightOnlyQuantOp(enum.IntEnum):
+    """gemv/weight_only_quant_op.h:12-18"""
+    UNDEFINED = 0
+    PER_COLUMN_SCALE_ONLY = 1
+    FINEGRAINED_SCALE_ONLY = 2
+    FINEGRAINED_SCALE_AND_ZEROS = 3
+
+
+class QuantType(enum.IntEnum):
+    """utils/type_base.h:7-11"""
+    W8_A16 = 0
+    W4_A16 = 1
+    W4_AFP8 = 2
+
+
+class LayoutType(enum.IntEnum):
+    """utils/type_base.h:13-16"""
+    kRowMajor = 0
+    kColumnMajor = 1
+
+
+def _host_ptr(a):
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def _dev_ptr(t):
+    if t is None:
+        return ctypes.c_void_p(0)
+    if isinstance(t, int):
+        return ctypes.c_void_p(t)
+    if hasattr(t, "data_ptr"):
+        if not t.is_cuda:
+            raise ValueError("device entry points need GPU tensors; there is no CPU path")
+        if not t.is_contiguous():
+            raise ValueError("tensors must be contiguous")
+        return ctypes.c_void_p(t.data_ptr())
+    raise TypeError(f"cannot take a device address from {type(t)!r}")
+
+
+def _stream_ptr(stream):
+    if stream is None:
+        import torch
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if isinstance(stream, int):
+        return ctypes.c_void_p(stream)
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _shape_arg(shape):
+    shape = [int(s) for s in shape]
+    return (ctypes.c_size_t * len(shape))(*shape), len(shape)
+
+
+class SubBytePacker:
+    """utils/preprocess.h:16-85 for <int4b_t, int8_t>."""
+
+    @staticmethod
+    def pack(unpacked):
+        unpacked = np.ascontiguousarray(unpacked, dtype=np.int8).reshape(-1)
+        packed = np.empty(unpacked.size // 2, dtype=np.uint8)
+        _lib.check(_lib.lib().mgemv_pack_int4(_host_ptr(packed), _host_ptr(unpacked), unpacked.size), "pack")
+        return packed
+
+    @staticmethod
+    def unpack(packed):
+        packed = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+        unpacked = np.empty(packed.size * 2, dtype=np.int8)
+        _lib.check(_lib.lib().mgemv_unpack_int4(_host_ptr(unpacked), _host_ptr(packed), packed.size), "unpack")
+        return unpacked
+
+
+class ZeroPointPreprocessor:
+    """utils/preprocess.h:88-102"""
+
+    @staticmethod
+    def neg_zero_point_multiplies_scale(scales, zeros):
+        s = np.ascontiguousarray(scales)
+        if s.dtype == np.float16:
+            s = s.view(np.uint16)
+        if s.dtype != np.uint16:
+            raise TypeError("scales must be float16 (or their uint16 bit patterns)")
+        z = np.ascontiguousarray(zeros, dtype=np.int8)
+        if z.size != s.size:
+            raise ValueError("scales and zeros differ in size")
+        out = np.empty(s.shape, dtype=np.uint16)
+        _lib.check(_lib.lib().mgemv_fold_zero_points(_host_ptr(out), _host_ptr(s), _host_ptr(z), s.size), "fold")
+        return out.view(np.float16)
+
+
+def preprocessed_size(shape, quant_type):
+    arr, rank = _shape_arg(shape)
+    return int(_lib.lib().mgemv_preprocessed_size(arr, rank, int(quant_type)))
+
+
+class MixedGemvWeightPreprocessor:
+    """utils/preprocess.h:480-524.  Same arguments; returns the preprocessed bytes (the
+    buffer may be larger than the input because rows and k are padded to whole tiles)."""
+
+    @staticmethod
+    def run(quantized_weight, shape, weight_layout=LayoutType.kColumnMajor, quant_type=QuantType.W4_A16,
+            force_interleave=False):
+        del force_interleave  # accepted and ignored, as in the reference (utils/preprocess.h:484)
+        src = np.ascontiguousarray(quantized_weight).reshape(-1).view(np.uint8)
+        arr, rank = _shape_arg(shape)
+        size = int(_lib.lib().mgemv_preprocessed_size(arr, rank, int(quant_type)))
+        if rank in (2, 3) and int(quant_type) in (0, 1):
+            n_elem = int(np.prod([int(s) for s in shape]))
+            need = n_elem * (4 if int(quant_type) == QuantType.W4_A16 else 8) // 8
+            if src.size < need:
+                raise ValueError(f"weight buffer holds {src.size} bytes, shape needs {need}")
+        dst = np.empty(max(size, 1), dtype=np.uint8)
+        _lib.check(_lib.lib().mgemv_preprocess_weights(_host_ptr(dst), _host_ptr(src), arr, rank,
+                                                       int(weight_layout), int(quant_type)), "preprocess")
+        return dst[:size]
+
+
+def unpreprocess_weights(preprocessed, shape, quant_type=QuantType.W4_A16):
+    src = np.ascontiguousarray(preprocessed, dtype=np.uint8).reshape(-1)
+    arr, rank = _shape_arg(shape)
+    n_elem = int(np.prod([int(s) for s in shape]))
+    bits = 4 if int(quant_type) == QuantType.W4_A16 else 8
+    dst = np.empty(n_elem * bits // 8, dtype=np.uint8)
+    _lib.check(_lib.lib().mgemv_unpreprocess_weights(_host_ptr(dst), _host_ptr(src), arr, rank, int(quant_type)),
+               "unpreprocess")
+    return dst
+
+
+def device_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, B, M, N, K, group_size,
+                quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, stream=None,
+                batch_strides=None):
+    """mixed_gemv_test.cu:124-165.  Reference letters: M = output features, N = activation
+    rows, K = reduction, B = batch count.  ptr_A is the PREPROCESSED weight buffer,
+    ptr_zero_point the folded fp16 term -z*s, ptr_C an optional fp16 bias.  The quant mode is
+    a run-time argument (a compile-time constant in the reference)."""
+    if B == 1 and not batch_strides:
+        st = _lib.lib().mgemv_gemv(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point),
+                                   _dev_ptr(ptr_C), _dev_ptr(ptr_D), int(M), int(N), int(K), int(group_size),
+                                   int(quant_op), int(weight_bits), _stream_ptr(stream))
+    else:
+        sa, sb, ss, sc, sd = batch_strides or (0, 0, 0, 0, 0)
+        st = _lib.lib().mgemv_gemv_batched(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale),
+                                           _dev_ptr(ptr_zero_point), _dev_ptr(ptr_C), _dev_ptr(ptr_D), int(B), int(M),
+                                           int(N), int(K), int(group_size), int(quant_op), int(weight_bits),
+                                           int(sa), int(sb), int(ss), int(sc), int(sd), _stream_ptr(stream))
+    _lib.check(st, "device_gemv")
+
+
+class GemvAdaptor:
+    """gemv/device/gemv_adaptor.h:114-261: Arguments / initialize / run / __call__."""
+
+    class Arguments:
+        def __init__(self, problem_size, ref_A, ref_B, ref_scale, ref_zero_point, ref_C, ref_D, group_size=64,
+                     batch_count=1, batch_stride_A=0, batch_stride_B=0, batch_stride_scale=0, batch_stride_C=0,
+                     batch_stride_D=0):
+            self.problem_size = tuple(int(v) for v in problem_size)  # (M, N, K)
+            self.ref_A, self.ref_B, self.ref_scale = ref_A, ref_B, ref_scale
+            self.ref_zero_point, self.ref_C, self.ref_D = ref_zero_point, ref_C, ref_D
+            self.group_size, self.batch_count = int(group_size), int(batch_count)
+            self.batch_strides = (batch_stride_A, batch_stride_B, batch_stride_scale, batch_stride_C, batch_stride_D)
+
+    def __init__(self, quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4):
+        self.quant_op, self.weight_bits = WeightOnlyQuantOp(quant_op), int(weight_bits)
+        self._args = None
+
+    def initialize(self, args, stream=None):
+        del stream
+        if self.quant_op != WeightOnlyQuantOp.PER_COLUMN_SCALE_ONLY and args.group_size < 64:
+            # gemv_adaptor.h:199-203 prints and exits; here it is an error
+            raise _lib.MixedGemvError(5, "GemvAdaptor.initialize")
+        self._args = args
+
+    def run(self, stream=None):
+        a = self._args
+        if a is None:
+            raise RuntimeError("GemvAdaptor.run before initialize")
+        m, n, k = a.problem_size
+        zero = a.ref_zero_point if self.quant_op == WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS else None
+        device_gemv(a.ref_A, a.ref_B, a.ref_scale, zero, a.ref_C, a.ref_D, a.batch_count, m, n, k, a.group_size,
+                    self.quant_op, self.weight_bits, stream,
+                    a.batch_strides if (a.batch_count != 1 or any(a.batch_strides)) else None)
+
+    def __call__(self, args, stream=None):
+        self.initialize(args, stream)
+        self.run(stream)
+
+
+def dequantize(ptr_A, ptr_scale, ptr_zero_point, ptr_out, M, K, group_size,
+               quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, stream=None):
+    """Writes dequantised weights [M][K] fp16 with the kernels' own converter + dequantiser."""
+    st = _lib.lib().mgemv_dequantize(_dev_ptr(ptr_A), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_out),
+                                     int(M), int(K), int(group_size), int(quant_op), int(weight_bits),
+                                     _stream_ptr(stream))
+    _lib.check(st, "dequantize")
+
+
+def set_launch_override(split_k_waves=0, tiles_per_workgroup=0):
+    _lib.check(_lib.lib().mgemv_set_launch_override(int(split_k_waves), int(tiles_per_workgroup)), "set_launch_override")
+
+
+def query_launch(n_out, m_batch, k, weight_bits=4):
+    out = (ctypes.c_int * 6)()
+    _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), ctypes.byref(out)),
+               "query_launch")
+    keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core")
+    return dict(zip(keys, list(out)))

@@ -1,0 +1,51 @@
+"""Builds the HIP library in-tree: mixed_gemv_amd/lib/libmixed_gemv_amd.so (gfx950 only)."""
+import os
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libmixed_gemv_amd.so")
+
+SOURCES = ["gemv_kernels.hip", "host_utils.cpp"]
+
+# -ffp-contract=off: the dequantiser is a separately rounded fp16 multiply and add.
+# -packed-fp32-ops off: keep the compiler from forming v_pk_*_f32.
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-fvisibility=hidden", "-DMGEMV_BUILDING_LIBRARY", "-fopenmp",
+    "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
+]
+
+
+def hipcc():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def build_library(verbose=True, extra_flags=()):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc(), *HIP_FLAGS, *extra_flags, "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC,
+               "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
+        objs.append(obj)
+    cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fopenmp", *objs, "-o", LIB_PATH]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library(extra_flags=tuple(sys.argv[1:]))

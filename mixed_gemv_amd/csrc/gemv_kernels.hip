@@ -1,0 +1,508 @@
+// GEMV and dequantise kernels for gfx950 (MI355X), wave64, plus their C-ABI launchers.
+//
+// One wavefront works on one 16-row tile of the weight matrix and a contiguous range of k
+// steps (units of tile_layout.h).  Per unit it issues four 1-KiB weight loads, one activation
+// load and the scale/zero loads, converts and dequantises in packed fp16 (two roundings, as
+// gemv/warp/warp_dequantizer.h:52-59), and accumulates in fp32 with v_dot2c_f32_f16 whose
+// activation operand is a DPP row broadcast.  Several waves of a workgroup split the k range
+// of the same tile (split-K); their per-lane partial sums meet in LDS, are summed in a fixed
+// order, biased, rounded to fp16 and stored.  This covers, for the reference, the main loops
+// of gemv/threadblock/dq_mma_singlestage_{finegrained,percol}.h, the reductions of
+// gemv/warp/reduce.h and gemv/threadblock/accumulator_combine.h, and the epilogue of
+// epilogue/threadblock/epilogue.h.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+
+#include "device_math.h"
+#include "mixed_gemv.h"
+#include "tile_layout.h"
+
+namespace mgemv {
+
+constexpr int kWave = 64;
+constexpr int kMaxWavesPerWorkgroup = 16;
+constexpr int kNumXcd = 8;
+constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
+
+struct GemvParams {
+  const uint8_t* weights;
+  const half_t* x;
+  const half_t* scale;
+  const half_t* zero_add;
+  const half_t* bias;
+  half_t* y;
+  int n_out;
+  int k;
+  int group_size;
+  int group_shift;     // log2(group_size) when it is a power of two, else -1
+  int num_groups;      // k / group_size (1 in per-column mode)
+  int tiles;           // ceil(n_out / 16)
+  int ksteps;          // ceil(k / kStepK)
+  int split_k;         // waves of a workgroup that share one tile       (blockDim.x / 64)
+  int tiles_per_wg;    //                                                  (blockDim.y)
+  int steps_per_wave;  // units per wave
+  int workgroups;      // logical workgroups per problem = ceil(tiles / tiles_per_wg)
+  int wgs_per_xcd;     // ceil(workgroups / 8); gridDim.x = 8 * wgs_per_xcd
+  long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
+};
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Neighbouring tiles read
+// neighbouring 32-byte pieces of the same scale/zero cache lines, so give each XCD (and its
+// private L2) a contiguous range of tiles instead of every eighth one.
+__device__ __forceinline__ int logical_workgroup(const GemvParams& p) {
+  const int xcd = blockIdx.x % kNumXcd;
+  const int slot = blockIdx.x / kNumXcd;
+  return xcd * p.wgs_per_xcd + slot;
+}
+
+__device__ __forceinline__ int group_of(const GemvParams& p, int k_index) {
+  int g = p.group_shift >= 0 ? (k_index >> p.group_shift) : (k_index / p.group_size);
+  return g < p.num_groups ? g : p.num_groups - 1;
+}
+
+// Everything one lane needs for one unit.
+template <int BITS, int MB, int GROUPS_PER_RUN>
+struct UnitFragment {
+  u32x4 w[kBlocksPerUnit];                       // 4 chunks of this lane's row
+  uint32_t x[MB][BITS == 4 ? 4 : 2];             // this lane's piece of the activation run
+  half_t s[GROUPS_PER_RUN], z[GROUPS_PER_RUN];   // scale / additive zero of the run
+};
+
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
+__device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f, const GemvParams& p,
+                                          __amdgpu_buffer_rsrc_t w_rsrc, const __amdgpu_buffer_rsrc_t (&x_rsrc)[MB],
+                                          int unit_in_wave, int kstep, int lane, int row) {
+  using G = Geometry<BITS>;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i)
+    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * kChunkBytes,
+                                                   unit_in_wave * kUnitBytes + i * kBlockBytes, kCacheStream);
+#pragma unroll
+  for (int m = 0; m < MB; ++m) {
+    if constexpr (BITS == 4) {
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc[m], lane * 16, kstep * (G::kStepK * 2), kCacheDefault);
+      f.x[m][0] = v[0]; f.x[m][1] = v[1]; f.x[m][2] = v[2]; f.x[m][3] = v[3];
+    } else {
+      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc[m], lane * 8, kstep * (G::kStepK * 2), kCacheDefault);
+      f.x[m][0] = v[0]; f.x[m][1] = v[1];
+    }
+  }
+  if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) {
+    const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
+      const int grp = group_of(p, k_run + gi * (G::kRunK / GROUPS_PER_RUN));
+      const int idx = grp * p.n_out + row;
+      f.s[gi] = p.scale[idx];
+      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS) f.z[gi] = p.zero_add[idx];
+    }
+  }
+}
+
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, int I>
+__device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
+                                              const ConvertRegs& c, half_t col_scale) {
+  constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  constexpr int gi = I * GROUPS_PER_RUN / kBlocksPerUnit;
+  const half2_t s2 = splat(QOP == MGEMV_PER_COLUMN_SCALE_ONLY ? col_scale : f.s[gi]);
+  const half2_t z2 = kHasZero ? splat(f.z[gi]) : half2_t{};
+  auto word = [&](auto J) {
+    constexpr int j = decltype(J)::value;
+    if constexpr (BITS == 4) {
+      half2_t q[4];
+      convert_int4_word(f.w[I][j], c, q);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) {
+        const half2_t d = dequant_pair<kHasZero>(q[h], s2, z2);
+#pragma unroll
+        for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + j>(acc[m], f.x[m][h], d);
+      }
+    } else {
+      half2_t q[2];
+      convert_int8_word(f.w[I][j], c, q);
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const half2_t d = dequant_pair<kHasZero>(q[h], s2, z2);
+#pragma unroll
+        for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + j>(acc[m], f.x[m][h], d);
+      }
+    }
+  };
+  word(std::integral_constant<int, 0>{});
+  word(std::integral_constant<int, 1>{});
+  word(std::integral_constant<int, 2>{});
+  word(std::integral_constant<int, 3>{});
+}
+
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
+__device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
+                                             const ConvertRegs& c, half_t col_scale) {
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 0>(acc, f, c, col_scale);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 1>(acc, f, c, col_scale);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 2>(acc, f, c, col_scale);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 3>(acc, f, c, col_scale);
+}
+
+// blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: tiles_per_wg * split_k * MB * 64 floats.
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
+__global__ void __launch_bounds__(kWave * kMaxWavesPerWorkgroup)
+gemv_dpp_kernel(const GemvParams p0) {
+  extern __shared__ float partials[];
+  GemvParams p = p0;
+  const int batch = blockIdx.z;
+  p.weights += batch * p.stride_weights;
+  p.x += batch * p.stride_x;
+  p.scale += batch * p.stride_scale;
+  if (p.zero_add) p.zero_add += batch * p.stride_scale;
+  if (p.bias) p.bias += batch * p.stride_bias;
+  p.y += batch * p.stride_y;
+
+  const int wg = logical_workgroup(p);
+  if (wg >= p.workgroups) return;  // whole workgroup leaves before any barrier
+
+  const int lane = threadIdx.x % kWave;
+  const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // position along k
+  const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);         // tile within the workgroup
+  const int tile = wg * p.tiles_per_wg + ty;
+  const int row_raw = tile * kTileRows + lane % kTileRows;
+  const int row = row_raw < p.n_out ? row_raw : p.n_out - 1;  // clamp padded rows (never stored)
+
+  float acc[MB];
+#pragma unroll
+  for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+
+  const int ks_begin = kw * p.steps_per_wave;
+  const int ks_end = min(ks_begin + p.steps_per_wave, p.ksteps);
+  if (tile < p.tiles && ks_begin < ks_end) {
+    const ConvertRegs c = make_convert_regs();
+    const int units = ks_end - ks_begin;
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
+        p.weights + ((size_t)tile * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
+        (uint32_t)units * (uint32_t)kUnitBytes);
+    __amdgpu_buffer_rsrc_t x_rsrc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) x_rsrc[m] = make_rsrc(p.x + (size_t)m * (size_t)p.k, (uint32_t)p.k * 2u);
+    half_t col_scale = (half_t)0.0f;
+    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = p.scale[row];
+
+    for (int u = 0; u < units; ++u) {
+      UnitFragment<BITS, MB, GROUPS_PER_RUN> f;
+      load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(f, p, w_rsrc, x_rsrc, u, ks_begin + u, lane, row);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, f, c, col_scale);
+    }
+#pragma unroll
+    for (int m = 0; m < MB; ++m) settle_dot_chain(acc[m]);
+  }
+
+  // Split-K / k-slice combine through LDS, fixed summation order.
+  const int slot = (ty * p.split_k + kw) * MB;
+#pragma unroll
+  for (int m = 0; m < MB; ++m) partials[(slot + m) * kWave + lane] = acc[m];
+  __syncthreads();
+
+  const int tid = threadIdx.y * blockDim.x + threadIdx.x;
+  const int nthreads = blockDim.x * blockDim.y;
+  const int outputs = p.tiles_per_wg * MB * kTileRows;
+  for (int o = tid; o < outputs; o += nthreads) {
+    const int r = o % kTileRows;
+    const int m = (o / kTileRows) % MB;
+    const int t = o / (kTileRows * MB);
+    const int n = (wg * p.tiles_per_wg + t) * kTileRows + r;
+    if (n >= p.n_out) continue;
+    float sum = 0.0f;
+    for (int w = 0; w < p.split_k; ++w) {
+      const float* part = partials + ((t * p.split_k + w) * MB + m) * kWave;
+#pragma unroll
+      for (int slice = 0; slice < kKSlices; ++slice) sum += part[slice * kTileRows + r];
+    }
+    // Epilogue: fp32 add of the bias, one rounding to fp16
+    // (host/mixed_gemv.h:102-103; epilogue/threadblock/epilogue.h:50-75).
+    if (p.bias) sum += (float)p.bias[n];
+    p.y[(size_t)m * (size_t)p.n_out + n] = (half_t)sum;
+  }
+}
+
+// One wave per unit; writes the dequantised weights of its 16 rows x kStepK columns.
+template <int BITS, int QOP>
+__global__ void __launch_bounds__(256) dequantize_kernel(const GemvParams p, half_t* __restrict__ out) {
+  using G = Geometry<BITS>;
+  constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  const int lane = threadIdx.x % kWave;
+  const long long unit = (long long)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (unit >= (long long)p.tiles * p.ksteps) return;
+  const int tile = (int)(unit / p.ksteps), kstep = (int)(unit % p.ksteps);
+  const int row = tile * kTileRows + lane % kTileRows;
+  const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
+  const ConvertRegs c = make_convert_regs();
+  const uint8_t* base = p.weights + (size_t)unit * kUnitBytes + (size_t)lane * kChunkBytes;
+  const int row_c = row < p.n_out ? row : p.n_out - 1;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) {
+    const int k0 = k_run + i * G::kChunkK;
+    const u32x4 w = *reinterpret_cast<const u32x4*>(base + i * kBlockBytes);
+    half_t s, z = (half_t)0.0f;
+    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+      s = p.scale[row_c];
+    } else {
+      const int idx = group_of(p, k0) * p.n_out + row_c;
+      s = p.scale[idx];
+      if constexpr (kHasZero) z = p.zero_add[idx];
+    }
+    const half2_t s2 = splat(s), z2 = splat(z);
+    if (row >= p.n_out || k0 >= p.k) continue;
+    half_t* dst = out + (size_t)row * (size_t)p.k + k0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (BITS == 4) {
+        half2_t q[4];
+        convert_int4_word(w[j], c, q);
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+          *reinterpret_cast<half2_t*>(dst + j * 8 + h * 2) = dequant_pair<kHasZero>(q[h], s2, z2);
+      } else {
+        half2_t q[2];
+        convert_int8_word(w[j], c, q);
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          *reinterpret_cast<half2_t*>(dst + j * 4 + h * 2) = dequant_pair<kHasZero>(q[h], s2, z2);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side: argument checks, launch geometry, dispatch
+// ---------------------------------------------------------------------------------------------
+
+std::atomic<int> g_override_split_k{0};
+std::atomic<int> g_override_tiles_per_wg{0};
+
+struct LaunchPlan {
+  int split_k, tiles_per_wg, steps_per_wave, workgroups, wgs_per_xcd, threads;
+};
+
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+LaunchPlan plan_launch(int n_out, int k, int bits) {
+  const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
+  // Aim for ~16 waves on each of the 256 compute units; a tile with few k steps cannot be
+  // split further than one unit per wave, and a workgroup holds at most 16 waves.
+  constexpr int kTargetWaves = 256 * 16;
+  int split_k = ceil_div(kTargetWaves, tiles);
+  const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
+  if (ov_sk > 0) split_k = ov_sk;
+  split_k = split_k < 1 ? 1 : split_k;
+  split_k = split_k > kMaxWavesPerWorkgroup ? kMaxWavesPerWorkgroup : split_k;
+  split_k = split_k > ksteps ? ksteps : split_k;
+  const int steps = ceil_div(ksteps, split_k);
+  split_k = ceil_div(ksteps, steps);
+  int tiles_per_wg = 4 / split_k;  // keep workgroups at >= 256 threads where the split allows
+  if (ov_tw > 0) tiles_per_wg = ov_tw;
+  if (tiles_per_wg < 1) tiles_per_wg = 1;
+  if (tiles_per_wg * split_k > kMaxWavesPerWorkgroup) tiles_per_wg = kMaxWavesPerWorkgroup / split_k;
+  LaunchPlan lp;
+  lp.split_k = split_k;
+  lp.tiles_per_wg = tiles_per_wg;
+  lp.steps_per_wave = steps;
+  lp.workgroups = ceil_div(tiles, tiles_per_wg);
+  lp.wgs_per_xcd = ceil_div(lp.workgroups, kNumXcd);
+  lp.threads = kWave * split_k * tiles_per_wg;
+  return lp;
+}
+
+int check_problem(const void* weights, const void* scale, const void* zero_add, int n_out, int k, int& group_size,
+                  int quant_op, int weight_bits) {
+  if (quant_op != MGEMV_PER_COLUMN_SCALE_ONLY && quant_op != MGEMV_FINEGRAINED_SCALE_ONLY &&
+      quant_op != MGEMV_FINEGRAINED_SCALE_AND_ZEROS)
+    return MGEMV_ERR_QUANT_OP;
+  if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
+  if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
+  if (n_out % 4) return MGEMV_ERR_ROWS;
+  if (k % chunk_k(weight_bits)) return MGEMV_ERR_COLS;
+  if (quant_op == MGEMV_PER_COLUMN_SCALE_ONLY) {
+    group_size = k;  // mixed_gemv_test.cu:142-143
+  } else {
+    if (group_size < 64) return MGEMV_ERR_GROUP_SIZE;  // gemv/device/gemv_adaptor.h:199-203
+    if (group_size % 32 || k % group_size) return MGEMV_ERR_GROUP_SIZE;
+  }
+  if (weights == nullptr || scale == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS && zero_add == nullptr) return MGEMV_ERR_NULL_POINTER;
+  // 32-bit index arithmetic inside the kernels
+  const long long groups = k / group_size;
+  if (groups * (long long)n_out >= (1ll << 30)) return MGEMV_ERR_SIZE;
+  if ((long long)num_ksteps(k, weight_bits) * kUnitBytes >= (1ll << 31)) return MGEMV_ERR_SIZE;
+  if ((long long)k * 2 * MGEMV_MAX_M_BATCH >= (1ll << 31)) return MGEMV_ERR_SIZE;
+  if (reinterpret_cast<uintptr_t>(weights) % 16) return MGEMV_ERR_ALIGNMENT;
+  if (reinterpret_cast<uintptr_t>(scale) % 2 || reinterpret_cast<uintptr_t>(zero_add) % 2) return MGEMV_ERR_ALIGNMENT;
+  return MGEMV_OK;
+}
+
+void fill_common(GemvParams& p, const void* weights, const uint16_t* scale, const uint16_t* zero_add, int n_out,
+                 int k, int group_size, int quant_op, int weight_bits) {
+  p = GemvParams{};
+  p.weights = static_cast<const uint8_t*>(weights);
+  p.scale = reinterpret_cast<const half_t*>(scale);
+  p.zero_add = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? reinterpret_cast<const half_t*>(zero_add) : nullptr;
+  p.n_out = n_out;
+  p.k = k;
+  p.group_size = group_size;
+  p.group_shift = (group_size & (group_size - 1)) == 0 ? __builtin_ctz((unsigned)group_size) : -1;
+  p.num_groups = k / group_size;
+  p.tiles = num_tiles(n_out);
+  p.ksteps = num_ksteps(k, weight_bits);
+}
+
+int groups_per_run(int group_size, int bits) {
+  const int run = run_k(bits);
+  if (group_size % run == 0) return 1;
+  if (group_size % (run / 2) == 0) return 2;
+  return 4;
+}
+
+template <int BITS, int QOP, int MB>
+hipError_t launch_gemv_gpr(const GemvParams& p, int gpr, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+  if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+    gemv_dpp_kernel<BITS, QOP, MB, 1><<<grid, block, lds, stream>>>(p);
+  } else {
+    switch (gpr) {
+      case 1: gemv_dpp_kernel<BITS, QOP, MB, 1><<<grid, block, lds, stream>>>(p); break;
+      case 2: gemv_dpp_kernel<BITS, QOP, MB, 2><<<grid, block, lds, stream>>>(p); break;
+      default: gemv_dpp_kernel<BITS, QOP, MB, 4><<<grid, block, lds, stream>>>(p); break;
+    }
+  }
+  return hipGetLastError();
+}
+
+template <int BITS, int QOP>
+hipError_t launch_gemv_mb(const GemvParams& p, int mb, int gpr, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+  switch (mb) {
+    case 1: return launch_gemv_gpr<BITS, QOP, 1>(p, gpr, grid, block, lds, stream);
+    case 2: return launch_gemv_gpr<BITS, QOP, 2>(p, gpr, grid, block, lds, stream);
+    case 3: return launch_gemv_gpr<BITS, QOP, 3>(p, gpr, grid, block, lds, stream);
+    default: return launch_gemv_gpr<BITS, QOP, 4>(p, gpr, grid, block, lds, stream);
+  }
+}
+
+hipError_t launch_gemv(const GemvParams& p, int bits, int qop, int mb, int gpr, dim3 grid, dim3 block, size_t lds,
+                       hipStream_t stream) {
+  if (bits == 4) {
+    switch (qop) {
+      case 1: return launch_gemv_mb<4, 1>(p, mb, gpr, grid, block, lds, stream);
+      case 2: return launch_gemv_mb<4, 2>(p, mb, gpr, grid, block, lds, stream);
+      default: return launch_gemv_mb<4, 3>(p, mb, gpr, grid, block, lds, stream);
+    }
+  }
+  switch (qop) {
+    case 1: return launch_gemv_mb<8, 1>(p, mb, gpr, grid, block, lds, stream);
+    case 2: return launch_gemv_mb<8, 2>(p, mb, gpr, grid, block, lds, stream);
+    default: return launch_gemv_mb<8, 3>(p, mb, gpr, grid, block, lds, stream);
+  }
+}
+
+template <int BITS>
+hipError_t launch_dequant(const GemvParams& p, int qop, half_t* out, hipStream_t stream) {
+  const long long units = (long long)p.tiles * p.ksteps;
+  const dim3 block(256), grid((unsigned)((units + 3) / 4));
+  switch (qop) {
+    case 1: dequantize_kernel<BITS, 1><<<grid, block, 0, stream>>>(p, out); break;
+    case 2: dequantize_kernel<BITS, 2><<<grid, block, 0, stream>>>(p, out); break;
+    default: dequantize_kernel<BITS, 3><<<grid, block, 0, stream>>>(p, out); break;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace mgemv
+
+extern "C" {
+
+int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+                       const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k,
+                       int group_size, int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x,
+                       int64_t stride_scale, int64_t stride_bias, int64_t stride_y, void* stream) {
+  using namespace mgemv;
+  if (batch_count < 1 || batch_count > 65535) return MGEMV_ERR_BATCH;
+  if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
+  if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
+  if (x == nullptr || y == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(y) % 2 ||
+      reinterpret_cast<uintptr_t>(bias) % 2)
+    return MGEMV_ERR_ALIGNMENT;
+  if (stride_weights % 16 || stride_x % 8) return MGEMV_ERR_ALIGNMENT;
+
+  GemvParams p;
+  fill_common(p, weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits);
+  p.bias = reinterpret_cast<const half_t*>(bias);
+  p.stride_weights = stride_weights;
+  p.stride_x = stride_x;
+  p.stride_scale = stride_scale;
+  p.stride_bias = stride_bias;
+  p.stride_y = stride_y;
+  const LaunchPlan lp = plan_launch(n_out, k, weight_bits);
+  p.split_k = lp.split_k;
+  p.tiles_per_wg = lp.tiles_per_wg;
+  p.steps_per_wave = lp.steps_per_wave;
+  p.workgroups = lp.workgroups;
+  p.wgs_per_xcd = lp.wgs_per_xcd;
+  const dim3 grid((unsigned)(lp.wgs_per_xcd * kNumXcd), 1, (unsigned)batch_count);
+  const dim3 block((unsigned)(kWave * lp.split_k), (unsigned)lp.tiles_per_wg, 1);
+  const int gpr = groups_per_run(group_size, weight_bits);
+
+  // Activation rows are processed kMaxValuBatch at a time.
+  for (int m0 = 0; m0 < m_batch; m0 += kMaxValuBatch) {
+    const int mb = m_batch - m0 < kMaxValuBatch ? m_batch - m0 : kMaxValuBatch;
+    GemvParams q = p;
+    q.x = reinterpret_cast<const half_t*>(x) + (size_t)m0 * (size_t)k;
+    q.y = reinterpret_cast<half_t*>(y) + (size_t)m0 * (size_t)n_out;
+    const size_t lds = (size_t)lp.tiles_per_wg * lp.split_k * mb * kWave * sizeof(float);
+    if (launch_gemv(q, weight_bits, quant_op, mb, gpr, grid, block, lds, static_cast<hipStream_t>(stream)) !=
+        hipSuccess)
+      return MGEMV_ERR_LAUNCH;
+  }
+  return MGEMV_OK;
+}
+
+int mgemv_gemv(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+               const uint16_t* bias, uint16_t* y, int n_out, int m_batch, int k, int group_size, int quant_op,
+               int weight_bits, void* stream) {
+  return mgemv_gemv_batched(weights, x, scale, zero_add, bias, y, 1, n_out, m_batch, k, group_size, quant_op,
+                            weight_bits, 0, 0, 0, 0, 0, stream);
+}
+
+int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t* zero_add, uint16_t* out, int n_out,
+                     int k, int group_size, int quant_op, int weight_bits, void* stream) {
+  using namespace mgemv;
+  if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
+  if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (reinterpret_cast<uintptr_t>(out) % 4) return MGEMV_ERR_ALIGNMENT;
+  GemvParams p;
+  fill_common(p, weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits);
+  const hipError_t e = weight_bits == 4
+                           ? launch_dequant<4>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream))
+                           : launch_dequant<8>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream));
+  return e == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+}
+
+int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup) {
+  if (split_k_waves < 0 || tiles_per_workgroup < 0) return MGEMV_ERR_SIZE;
+  mgemv::g_override_split_k.store(split_k_waves);
+  mgemv::g_override_tiles_per_wg.store(tiles_per_workgroup);
+  return MGEMV_OK;
+}
+
+int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[6]) {
+  if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
+  if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
+  if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
+  const mgemv::LaunchPlan lp = mgemv::plan_launch(n_out, k, weight_bits);
+  out[0] = lp.wgs_per_xcd * mgemv::kNumXcd;
+  out[1] = lp.threads;
+  out[2] = lp.split_k;
+  out[3] = lp.tiles_per_wg;
+  out[4] = lp.steps_per_wave;
+  out[5] = 0;
+  return MGEMV_OK;
+}
+
+}  // extern "C"

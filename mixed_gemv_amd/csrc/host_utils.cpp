@@ -1,0 +1,252 @@
+// Host-side utilities of the library: int4 packing, zero-point folding and the weight
+// preprocessor that produces the gfx950 tile layout.  They stand in for
+// utils/preprocess.h:41-84 (SubBytePacker), :94-101 (ZeroPointPreprocessor) and :482-522
+// (MixedGemvWeightPreprocessor::run) of the reference: same inputs, same meaning, new layout.
+#include <cstring>
+#include <vector>
+
+#include "mixed_gemv.h"
+#include "tile_layout.h"
+
+namespace {
+
+// ---- binary16 helpers (host) ---------------------------------------------------------------
+
+inline uint32_t bits_of(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  return u;
+}
+inline float float_of(uint32_t u) {
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+// Exact widening binary16 -> binary32 through a power-of-two rescale.
+inline float half_bits_to_float(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  const uint32_t body = (uint32_t)(h & 0x7fffu);
+  if (body >= 0x7c00u) return float_of(sign | 0x7f800000u | ((body & 0x3ffu) << 13));
+  // Place exponent+mantissa in the binary32 fields, then multiply by 2^(127-15) = 2^112:
+  // exact for normals, and it normalises subnormals for free.
+  const float scaled = float_of(body << 13) * float_of(0x77800000u);
+  return float_of(sign | bits_of(scaled));
+}
+
+// binary32 -> binary16, round-to-nearest-even.
+inline uint16_t float_to_half_bits(float f) {
+  uint32_t x = bits_of(f);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  x &= 0x7fffffffu;
+  if (x >= 0x47800000u) {  // |f| >= 65536, inf or nan
+    return (uint16_t)(sign | (x > 0x7f800000u ? 0x7e00u : 0x7c00u));
+  }
+  if (x < 0x38800000u) {  // |f| < 2^-14: the result is subnormal (or zero)
+    // Adding 0.5 shifts the value so that the binary32 unit in the last place is 2^-24,
+    // the subnormal half spacing; the hardware's RNE does the rounding.
+    const float shifted = float_of(x) + 0.5f;
+    return (uint16_t)(sign | (bits_of(shifted) - 0x3f000000u));
+  }
+  const uint32_t odd = (x >> 13) & 1u;
+  x += 0xc8000fffu;  // rebias exponent by (15 - 127) and add the rounding bias 0xfff
+  x += odd;          // ties go to even
+  return (uint16_t)(sign | (x >> 13));
+}
+
+bool shape_ok(const size_t* shape, int rank, size_t& experts, size_t& k, size_t& n_out) {
+  if (shape == nullptr || (rank != 2 && rank != 3)) return false;
+  experts = rank == 2 ? 1 : shape[0];
+  k = rank == 2 ? shape[0] : shape[1];
+  n_out = rank == 2 ? shape[1] : shape[2];
+  return true;
+}
+
+int bits_of_quant_type(int quant_type) {
+  if (quant_type == MGEMV_W4_A16) return 4;
+  if (quant_type == MGEMV_W8_A16) return 8;
+  return 0;
+}
+
+// Transpose a [k][n_out] matrix of `bits`-wide elements into [n_out][k] (both densely packed,
+// low nibble = even index).  Blocked so that both sides are walked in cache-sized tiles.
+void transpose_quantised(uint8_t* dst, const uint8_t* src, size_t k, size_t n_out, int bits) {
+  constexpr size_t kBlock = 64;
+  if (bits == 8) {
+    for (size_t k0 = 0; k0 < k; k0 += kBlock)
+      for (size_t n0 = 0; n0 < n_out; n0 += kBlock) {
+        const size_t k1 = k0 + kBlock < k ? k0 + kBlock : k;
+        const size_t n1 = n0 + kBlock < n_out ? n0 + kBlock : n_out;
+        for (size_t n = n0; n < n1; ++n)
+          for (size_t kk = k0; kk < k1; ++kk) dst[n * k + kk] = src[kk * n_out + n];
+      }
+    return;
+  }
+  std::memset(dst, 0, n_out * k / 2);
+  for (size_t k0 = 0; k0 < k; k0 += kBlock)
+    for (size_t n0 = 0; n0 < n_out; n0 += kBlock) {
+      const size_t k1 = k0 + kBlock < k ? k0 + kBlock : k;
+      const size_t n1 = n0 + kBlock < n_out ? n0 + kBlock : n_out;
+      for (size_t n = n0; n < n1; ++n)
+        for (size_t kk = k0; kk < k1; ++kk) {
+          const size_t si = kk * n_out + n;
+          const uint8_t v = (uint8_t)((src[si >> 1] >> (4 * (si & 1))) & 0xfu);
+          const size_t di = n * k + kk;
+          dst[di >> 1] = (uint8_t)(dst[di >> 1] | (v << (4 * (di & 1))));
+        }
+    }
+}
+
+// One matrix: rows of k elements (n_out rows) -> tile layout.
+void tile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k, int bits) {
+  const size_t ksteps = (size_t)mgemv::num_ksteps((int)k, bits);
+  const size_t ck = (size_t)mgemv::chunk_k(bits);
+  const size_t row_bytes = k * (size_t)bits / 8;
+  std::memset(dst, 0, mgemv::preprocessed_bytes(n_out, k, bits));
+#pragma omp parallel for schedule(static)
+  for (long long n = 0; n < (long long)n_out; ++n) {
+    const uint8_t* row = src + (size_t)n * row_bytes;
+    for (size_t k0 = 0; k0 < k; k0 += ck) {
+      uint32_t words[4];
+      std::memcpy(words, row + k0 * (size_t)bits / 8, mgemv::kChunkBytes);
+      for (int j = 0; j < 4; ++j)
+        words[j] = bits == 4 ? mgemv::encode_int4_word(words[j]) : mgemv::encode_int8_word(words[j]);
+      std::memcpy(dst + mgemv::chunk_offset((size_t)n, k0, ksteps, bits), words, mgemv::kChunkBytes);
+    }
+  }
+}
+
+void untile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k, int bits) {
+  const size_t ksteps = (size_t)mgemv::num_ksteps((int)k, bits);
+  const size_t ck = (size_t)mgemv::chunk_k(bits);
+  const size_t row_bytes = k * (size_t)bits / 8;
+#pragma omp parallel for schedule(static)
+  for (long long n = 0; n < (long long)n_out; ++n) {
+    uint8_t* row = dst + (size_t)n * row_bytes;
+    for (size_t k0 = 0; k0 < k; k0 += ck) {
+      uint32_t words[4];
+      std::memcpy(words, src + mgemv::chunk_offset((size_t)n, k0, ksteps, bits), mgemv::kChunkBytes);
+      for (int j = 0; j < 4; ++j)
+        words[j] = bits == 4 ? mgemv::decode_int4_word(words[j]) : mgemv::decode_int8_word(words[j]);
+      std::memcpy(row + k0 * (size_t)bits / 8, words, mgemv::kChunkBytes);
+    }
+  }
+}
+
+int check_dims(size_t n_out, size_t k, int bits) {
+  if (n_out == 0 || k == 0) return MGEMV_ERR_SIZE;
+  if (n_out % 4) return MGEMV_ERR_ROWS;                          // utils/preprocess.h:319-322
+  if (k % (size_t)mgemv::chunk_k(bits)) return MGEMV_ERR_COLS;   // one 128-bit access of one row
+  if (n_out > 0x7fffffffull || k > 0x7fffffffull) return MGEMV_ERR_SIZE;
+  return MGEMV_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mgemv_pack_int4(uint8_t* packed, const int8_t* unpacked, size_t n_unpacked) {
+  if (n_unpacked == 0) return MGEMV_OK;
+  if (packed == nullptr || unpacked == nullptr) return MGEMV_ERR_NULL_POINTER;
+  const size_t n_bytes = n_unpacked / 2;
+  for (size_t i = 0; i < n_bytes; ++i) {
+    const unsigned lo = (unsigned)unpacked[2 * i] & 0xfu;
+    const unsigned hi = (unsigned)unpacked[2 * i + 1] & 0xfu;
+    packed[i] = (uint8_t)(lo | (hi << 4));
+  }
+  return MGEMV_OK;
+}
+
+int mgemv_unpack_int4(int8_t* unpacked, const uint8_t* packed, size_t n_packed) {
+  if (n_packed == 0) return MGEMV_OK;
+  if (packed == nullptr || unpacked == nullptr) return MGEMV_ERR_NULL_POINTER;
+  for (size_t i = 0; i < n_packed; ++i) {
+    const int lo = packed[i] & 0xf, hi = packed[i] >> 4;
+    unpacked[2 * i] = (int8_t)(lo >= 8 ? lo - 16 : lo);
+    unpacked[2 * i + 1] = (int8_t)(hi >= 8 ? hi - 16 : hi);
+  }
+  return MGEMV_OK;
+}
+
+int mgemv_fold_zero_points(uint16_t* out, const uint16_t* scales, const int8_t* zeros, size_t n) {
+  if (n == 0) return MGEMV_OK;
+  if (out == nullptr || scales == nullptr || zeros == nullptr) return MGEMV_ERR_NULL_POINTER;
+  for (size_t i = 0; i < n; ++i) {
+    // -z is an integer of magnitude <= 128: exact in binary16.  The binary32 product of two
+    // halves is exact, so one rounding to binary16 is the correctly rounded fp16 multiply.
+    const float neg_z = (float)(-(int)zeros[i]);
+    out[i] = float_to_half_bits(neg_z * half_bits_to_float(scales[i]));
+  }
+  return MGEMV_OK;
+}
+
+size_t mgemv_preprocessed_size(const size_t* shape, int rank, int quant_type) {
+  size_t experts, k, n_out;
+  const int bits = bits_of_quant_type(quant_type);
+  if (bits == 0 || !shape_ok(shape, rank, experts, k, n_out)) return 0;
+  return experts * mgemv::preprocessed_bytes(n_out, k, bits);
+}
+
+int mgemv_preprocess_weights(uint8_t* dst, const uint8_t* src, const size_t* shape, int rank, int layout,
+                             int quant_type) {
+  if (dst == nullptr || src == nullptr || shape == nullptr) return MGEMV_ERR_NULL_POINTER;
+  size_t experts, k, n_out;
+  if (!shape_ok(shape, rank, experts, k, n_out)) return MGEMV_ERR_RANK;
+  const int bits = bits_of_quant_type(quant_type);
+  if (bits == 0) return MGEMV_ERR_QUANT_TYPE;
+  if (layout != MGEMV_ROW_MAJOR && layout != MGEMV_COLUMN_MAJOR) return MGEMV_ERR_LAYOUT;
+  if (const int st = check_dims(n_out, k, bits)) return st;
+
+  const size_t src_bytes = n_out * k * (size_t)bits / 8;
+  const size_t dst_bytes = mgemv::preprocessed_bytes(n_out, k, bits);
+  std::vector<uint8_t> transposed;
+  if (layout == MGEMV_ROW_MAJOR) transposed.resize(src_bytes);
+  for (size_t e = 0; e < experts; ++e) {
+    const uint8_t* matrix = src + e * src_bytes;
+    if (layout == MGEMV_ROW_MAJOR) {
+      transpose_quantised(transposed.data(), matrix, k, n_out, bits);
+      matrix = transposed.data();
+    }
+    tile_one_matrix(dst + e * dst_bytes, matrix, n_out, k, bits);
+  }
+  return MGEMV_OK;
+}
+
+int mgemv_unpreprocess_weights(uint8_t* dst, const uint8_t* src_preprocessed, const size_t* shape, int rank,
+                               int quant_type) {
+  if (dst == nullptr || src_preprocessed == nullptr || shape == nullptr) return MGEMV_ERR_NULL_POINTER;
+  size_t experts, k, n_out;
+  if (!shape_ok(shape, rank, experts, k, n_out)) return MGEMV_ERR_RANK;
+  const int bits = bits_of_quant_type(quant_type);
+  if (bits == 0) return MGEMV_ERR_QUANT_TYPE;
+  if (const int st = check_dims(n_out, k, bits)) return st;
+  const size_t raw_bytes = n_out * k * (size_t)bits / 8;
+  const size_t tiled_bytes = mgemv::preprocessed_bytes(n_out, k, bits);
+  for (size_t e = 0; e < experts; ++e)
+    untile_one_matrix(dst + e * raw_bytes, src_preprocessed + e * tiled_bytes, n_out, k, bits);
+  return MGEMV_OK;
+}
+
+const char* mgemv_status_string(int status) {
+  switch (status) {
+    case MGEMV_OK: return "ok";
+    case MGEMV_ERR_NULL_POINTER: return "a required pointer is NULL";
+    case MGEMV_ERR_RANK: return "weight shape must be 2-D {k, n_out} or 3-D {experts, k, n_out}";
+    case MGEMV_ERR_ROWS: return "n_out must be a multiple of 4";
+    case MGEMV_ERR_COLS: return "k must be a multiple of one 128-bit weight access (32 int4 / 16 int8 elements)";
+    case MGEMV_ERR_GROUP_SIZE: return "group_size must be >= 64, a multiple of 32 and divide k";
+    case MGEMV_ERR_QUANT_OP: return "quant_op must be 1 (per-column scale), 2 (group scale) or 3 (group scale + zero)";
+    case MGEMV_ERR_QUANT_TYPE: return "weights must be int8 (W8_A16) or int4 (W4_A16)";
+    case MGEMV_ERR_BATCH: return "batch_count must be >= 1 and m_batch in [1, 16]";
+    case MGEMV_ERR_LAYOUT: return "layout must be 0 (row major) or 1 (column major)";
+    case MGEMV_ERR_SIZE: return "a dimension is zero, negative or exceeds the 32-bit index range of the kernels";
+    case MGEMV_ERR_LAUNCH: return "HIP launch failed";
+    case MGEMV_ERR_NO_DEVICE: return "no usable gfx950 device";
+    case MGEMV_ERR_ALIGNMENT: return "device pointer alignment: weights and activations 16 bytes, scales/zeros/bias/output 8 bytes";
+    default: return "unknown status";
+  }
+}
+
+int mgemv_version(void) { return 100; }
+
+}  // extern "C"

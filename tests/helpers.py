@@ -1,0 +1,99 @@
+"""Shared test helpers: seeded problems (from the oracle's generator) and error metrics."""
+import numpy as np
+
+import oracle as orc
+
+PER_COLUMN, SCALE_ONLY, SCALE_AND_ZEROS = 1, 2, 3
+
+
+def seed_of(tag, tensor, buffer=0):
+    """One documented 64-bit seed per (problem tag, tensor, buffer)."""
+    h = 1469598103934665603
+    for ch in f"{tag}/{tensor}/{buffer}".encode():
+        h = ((h ^ ch) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+class Problem:
+    """Raw (un-preprocessed) operands of one GEMV, as numpy arrays."""
+
+    def __init__(self, tag, n_out, k, bits, quant_op, group_size, m_batch=1, bias=False, x_dist="uniform",
+                 scale_range=(0.001, 0.02), zero_kind="f16", zero_range=(-0.05, 0.05), buffer=0):
+        self.tag, self.n_out, self.k, self.bits, self.quant_op = tag, n_out, k, bits, quant_op
+        self.group_size = k if quant_op == PER_COLUMN else group_size
+        self.m_batch = m_batch
+        groups = k // self.group_size
+        lo, hi = (-8, 7) if bits == 4 else (-128, 127)
+        self.q = orc.fill_int8(n_out * k, seed_of(tag, "w", buffer), lo, hi)
+        self.w_raw = orc.pack_int4(self.q) if bits == 4 else self.q.view(np.uint8).copy()
+        if x_dist == "uniform":
+            self.x = orc.fill_uniform_f16(m_batch * k, seed_of(tag, "x"), -1.0, 1.0).reshape(m_batch, k)
+        else:
+            self.x = orc.fill_normal_clipped_f16(m_batch * k, seed_of(tag, "x"), 4.0).reshape(m_batch, k)
+        self.scale = orc.fill_uniform_f16(groups * n_out, seed_of(tag, "s", buffer), *scale_range).reshape(groups, n_out)
+        self.zeros_i8 = None
+        self.zero_add = None
+        if quant_op == SCALE_AND_ZEROS:
+            if zero_kind == "int8":
+                self.zeros_i8 = orc.fill_int8(groups * n_out, seed_of(tag, "z", buffer), -8, 7).reshape(groups, n_out)
+                self.zero_add = orc.fold_zero_points(self.scale, self.zeros_i8)
+            else:
+                self.zero_add = orc.fill_uniform_f16(groups * n_out, seed_of(tag, "z", buffer), *zero_range).reshape(
+                    groups, n_out)
+        self.bias = orc.fill_uniform_f16(n_out, seed_of(tag, "b"), -0.1, 0.1) if bias else None
+
+    def oracle_dequant(self):
+        return orc.dequantize(self.w_raw, self.scale, self.zero_add, self.n_out, self.k, self.group_size,
+                              self.quant_op, self.bits)
+
+    def oracle_gemv(self, threads=8, literal_int8_zero=False):
+        zero = self.zeros_i8 if (literal_int8_zero and self.zeros_i8 is not None) else self.zero_add
+        return orc.gemv(self.w_raw, self.x, self.scale, zero, self.bias, self.n_out, self.m_batch, self.k,
+                        self.group_size, self.quant_op, self.bits, threads=threads)
+
+
+def error_report(got, ref):
+    """max abs error, and max relative error with denominator max(|ref|, 2^-10 * rms(ref))."""
+    g = np.asarray(got, dtype=np.float64).reshape(-1)
+    r = np.asarray(ref, dtype=np.float64).reshape(-1)
+    rms = float(np.sqrt(np.mean(r * r))) if r.size else 0.0
+    floor = max(rms * 2.0 ** -10, 2.0 ** -24)
+    abs_err = np.abs(g - r)
+    rel = abs_err / np.maximum(np.abs(r), floor)
+    return float(abs_err.max(initial=0.0)), float(rel.max(initial=0.0)), floor
+
+
+class DeviceProblem:
+    """Uploads a Problem through the library's own preprocessor."""
+
+    def __init__(self, prob, device):
+        import torch
+        import mixed_gemv_amd as mg
+        self.p = prob
+        qt = mg.QuantType.W4_A16 if prob.bits == 4 else mg.QuantType.W8_A16
+        pre = mg.MixedGemvWeightPreprocessor.run(prob.w_raw, (prob.k, prob.n_out), mg.LayoutType.kColumnMajor, qt)
+        self.w = torch.from_numpy(pre).to(device)
+        self.x = torch.from_numpy(prob.x.view(np.int16)).to(device)
+        self.scale = torch.from_numpy(prob.scale.view(np.int16)).to(device)
+        self.zero = torch.from_numpy(prob.zero_add.view(np.int16)).to(device) if prob.zero_add is not None else None
+        self.bias = torch.from_numpy(prob.bias.view(np.int16)).to(device) if prob.bias is not None else None
+        self.y = torch.zeros((prob.m_batch, prob.n_out), dtype=torch.int16, device=device)
+
+    def run(self):
+        import torch
+        import mixed_gemv_amd as mg
+        p = self.p
+        self.y.fill_(0x7e00)  # NaN pattern: every output must be overwritten
+        mg.device_gemv(self.w, self.x, self.scale, self.zero, self.bias, self.y, 1, p.n_out, p.m_batch, p.k,
+                       p.group_size, p.quant_op, p.bits)
+        torch.cuda.synchronize()
+        return self.y.cpu().numpy().view(np.float16)
+
+    def dequant(self):
+        import torch
+        import mixed_gemv_amd as mg
+        p = self.p
+        out = torch.zeros((p.n_out, p.k), dtype=torch.int16, device=self.w.device)
+        mg.dequantize(self.w, self.scale, self.zero, out, p.n_out, p.k, p.group_size, p.quant_op, p.bits)
+        torch.cuda.synchronize()
+        return out.cpu().numpy().view(np.float16)
