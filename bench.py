@@ -1,0 +1,276 @@
+#!/usr/bin/env python3
+"""Benchmark of the weight-only-quantised GEMV hot path on one MI355X.
+
+A step is one GEMV call (one pass of the hot path over one activation batch).  Operands are
+synthetic, seeded, and already resident in HBM when the timed region starts; weight / scale /
+zero buffers are rotated between calls so that more than the 256 MB Infinity Cache is
+touched between two uses of the same buffer (cold-cache timing).
+
+Prints ONE JSON line:
+  value            whole-job algorithmic GB/s over the K timed steps (wall clock, launch gaps included)
+  roofline         achieved = algorithmic bytes per launch / average kernel duration, measured with a
+                   HIP event pair on the launch stream around the back-to-back launches of the timed
+                   region (gaps between kernels count as kernel time); peak = 8000 GB/s
+  cpu_baseline     the CPU oracle (a port of the reference's HOST_CHECK loop) timed on this host
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBS = 8000.0
+MALL_BYTES = 256 << 20
+
+# name -> (n_out, k, weight_bits, quant_op, group_size, m_batch, bias, x distribution, scale range, description)
+WORKLOADS = {
+    "ns": (4096, 4096, 4, 3, 128, 1, False, "uniform", (0.001, 0.02),
+           "int4 group-128 scale+zero GEMV, M=1, N=K=4096"),
+    "c1": (4096, 4096, 8, 1, 4096, 1, True, "uniform", (0.001, 0.01),
+           "int8 per-column scale GEMV + bias, M=1, N=K=4096"),
+    "c2": (4096, 4096, 4, 2, 128, 1, True, "uniform", (0.001, 0.02),
+           "int4 group-128 scale-only GEMV + bias, M=1, N=K=4096"),
+    "c3a": (11008, 4096, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
+            "int4 group-128 scale+zero GEMV, M=1, K=4096, N=11008"),
+    "c3b": (4096, 11008, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
+            "int4 group-128 scale+zero GEMV, M=1, K=11008, N=4096"),
+    "c4": (8192, 8192, 4, 3, 64, 1, True, "uniform", (0.001, 0.02),
+           "int4 group-64 scale+zero GEMV + bias, N=K=8192"),
+    "c5": (28672, 8192, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
+           "int4 group-128 scale+zero GEMV, M=1, K=8192, N=28672"),
+}
+
+
+def algorithmic_bytes(n_out, k, bits, quant_op, group, m_batch, bias):
+    groups = 1 if quant_op == 1 else k // group
+    return (n_out * k * bits // 8 + groups * n_out * 2 * (2 if quant_op == 3 else 1) + (n_out * 2 if bias else 0)
+            + m_batch * k * 2 + m_batch * n_out * 2)
+
+
+class Workload:
+    """Builds the rotating operand sets of one workload directly in HBM (torch is the allocator)."""
+
+    def __init__(self, name, device, m_batch=None, seed=1234, min_sets=None):
+        import numpy as np
+        import torch
+        import mixed_gemv_amd as mg
+
+        (self.n_out, self.k, self.bits, self.quant_op, self.group, mb, self.has_bias, xdist, srange,
+         self.description) = WORKLOADS[name]
+        self.name = name
+        self.m_batch = m_batch or mb
+        self.bytes = algorithmic_bytes(self.n_out, self.k, self.bits, self.quant_op, self.group, self.m_batch,
+                                       self.has_bias)
+        groups = 1 if self.quant_op == 1 else self.k // self.group
+        per_set = self.n_out * self.k * self.bits // 8 + 2 * groups * self.n_out * 2
+        # enough sets that (sets - 1) * per_set exceeds the Infinity Cache plus the 8 x 4 MB L2s
+        self.sets = max(2, -(-(MALL_BYTES + (32 << 20)) // per_set) + 1)
+        if min_sets:
+            self.sets = max(self.sets, min_sets)
+        gen = torch.Generator(device="cpu").manual_seed(seed)
+        qt = mg.QuantType.W4_A16 if self.bits == 4 else mg.QuantType.W8_A16
+        self.raw0 = None
+        self.w, self.s, self.z = [], [], []
+        for i in range(self.sets):
+            # uniform random bytes == uniform int4 pairs in [-8, 7] (or int8 in [-128, 127])
+            raw = torch.randint(0, 256, (self.n_out * self.k * self.bits // 8,), dtype=torch.uint8, generator=gen)
+            if i == 0:
+                self.raw0 = raw.numpy().copy()
+            pre = mg.MixedGemvWeightPreprocessor.run(raw.numpy(), (self.k, self.n_out), mg.LayoutType.kColumnMajor, qt)
+            self.w.append(torch.from_numpy(pre).to(device))
+            sc = (torch.rand((groups, self.n_out), generator=gen) * (srange[1] - srange[0]) + srange[0]).half()
+            self.s.append(sc.to(device))
+            if self.quant_op == 3:
+                zz = (torch.rand((groups, self.n_out), generator=gen) * 0.1 - 0.05).half()
+                self.z.append(zz.to(device))
+            else:
+                self.z.append(None)
+        if xdist == "uniform":
+            x = torch.rand((self.m_batch, self.k), generator=gen) * 2 - 1
+        else:
+            x = torch.randn((self.m_batch, self.k), generator=gen).clamp_(-4, 4)
+        self.x = x.half().to(device)
+        self.bias = (torch.rand((self.n_out,), generator=gen) * 0.2 - 0.1).half().to(device) if self.has_bias else None
+        self.y = torch.zeros((self.m_batch, self.n_out), dtype=torch.half, device=device)
+        self.np = np
+        self.mg = mg
+
+    def launch(self, i):
+        j = i % self.sets
+        self.mg.device_gemv(self.w[j], self.x, self.s[j], self.z[j], self.bias, self.y, 1, self.n_out, self.m_batch,
+                            self.k, self.group, self.quant_op, self.bits)
+
+    def host_operands(self, j=0):
+        np = self.np
+        return dict(
+            w_raw=self.raw0 if j == 0 else None,
+            x=self.x.cpu().numpy(), scale=self.s[j].cpu().numpy(),
+            zero=self.z[j].cpu().numpy() if self.z[j] is not None else None,
+            bias=self.bias.cpu().numpy() if self.bias is not None else None)
+
+
+def time_workload(wl, steps, warmup, use_graph=False):
+    """Returns (wall seconds for `steps` steps, average kernel microseconds by HIP events)."""
+    import torch
+    for i in range(warmup):
+        wl.launch(i)
+    torch.cuda.synchronize()
+    graph = None
+    if use_graph:
+        # one rotation of the buffer sets captured once, replayed; launches only, no memsets
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(wl.sets):
+                    wl.launch(i)
+        torch.cuda.current_stream().wait_stream(side)
+        graph.replay()
+        torch.cuda.synchronize()
+        replays = max(1, steps // wl.sets)
+        steps = replays * wl.sets
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    if graph is not None:
+        for _ in range(replays):
+            graph.replay()
+    else:
+        for i in range(steps):
+            wl.launch(i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, e0.elapsed_time(e1) * 1e3 / steps, steps
+
+
+def check_against_oracle(wl, rows=None):
+    """GPU result of buffer set 0 against the CPU oracle on the first `rows` rows; also times
+    the oracle single-threaded (the reference's HOST_CHECK loop has no threading)."""
+    import numpy as np
+    import torch
+    import oracle as orc  # cpu_baseline leg: the checker, never the thing measured
+
+    ops = wl.host_operands(0)
+    rows = wl.n_out if rows is None else min(rows, wl.n_out)
+    row_bytes = wl.k * wl.bits // 8
+    w_rows = np.ascontiguousarray(ops["w_raw"][: rows * row_bytes])
+    if wl.bits == 8:
+        w_rows = w_rows.view(np.int8)
+    scale = np.ascontiguousarray(ops["scale"][:, :rows])
+    zero = np.ascontiguousarray(ops["zero"][:, :rows]) if ops["zero"] is not None else None
+    bias = np.ascontiguousarray(ops["bias"][:rows]) if ops["bias"] is not None else None
+    reps, elapsed, ref = 0, 0.0, None
+    while reps < 2 or (elapsed < 8.0 and reps < 64):
+        t0 = time.perf_counter()
+        ref = orc.gemv(w_rows, ops["x"], scale, zero, bias, rows, wl.m_batch, wl.k, wl.group, wl.quant_op, wl.bits,
+                       threads=1)
+        elapsed += time.perf_counter() - t0
+        reps += 1
+    cpu_s = elapsed / reps
+    wl.launch(0)
+    torch.cuda.synchronize()
+    got = wl.y.cpu().numpy()[:, :rows].astype(np.float64)
+    r = ref.astype(np.float64)
+    rms = float(np.sqrt(np.mean(r * r)))
+    floor = max(rms * 2.0 ** -10, 2.0 ** -24)
+    abs_err = np.abs(got - r)
+    rel_err = abs_err / np.maximum(np.abs(r), floor)
+    sample_bytes = algorithmic_bytes(rows, wl.k, wl.bits, wl.quant_op, wl.group, wl.m_batch, wl.has_bias)
+    return dict(cpu_seconds=cpu_s, cpu_reps=reps, sample_bytes=sample_bytes, rows=rows,
+                max_abs_err=float(abs_err.max()), max_rel_err=float(rel_err.max()), rel_floor=floor)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=4000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--workload", default="ns", choices=sorted(WORKLOADS))
+    ap.add_argument("--m-batch", type=int, default=None)
+    ap.add_argument("--launch", default="graph", choices=["graph", "stream"],
+                    help="graph: the steps are replayed from a captured HIP graph (one kernel node per step, one "
+                         "rotation of the buffer sets per replay); stream: one host launch per step")
+    ap.add_argument("--extra", default="c5", help="comma list of further workloads reported under 'other_workloads' ('' = none)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / oracle check")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (a GEMV over one weight matrix held by one MI355X); "
+              "--gpus above 1 is not supported", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    import mixed_gemv_amd as mg
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    wl = Workload(args.workload, device, m_batch=args.m_batch)
+    wall, ev_us, steps = time_workload(wl, args.steps, args.warmup, use_graph=(args.launch == "graph"))
+    us_per_step = wall * 1e6 / steps
+    value = wl.bytes / (wall / steps) / 1e9
+    kernel_us = ev_us
+    achieved = wl.bytes / (kernel_us * 1e-6) / 1e9
+    plan = mg.query_launch(wl.n_out, wl.m_batch, wl.k, wl.bits)
+
+    out = {
+        "metric": "HBM GB/s & % of peak, us/call; int4-g128 GEMV M=1, N=K=4096",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(us_per_step / 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": wl.description, "name": wl.name, "n_out": wl.n_out, "k": wl.k, "m_batch": wl.m_batch,
+                   "weight_bits": wl.bits, "quant_op": wl.quant_op, "group_size": wl.group, "bias": wl.has_bias,
+                   "buffer_sets_rotated": wl.sets, "launch": "hip_graph" if args.launch == "graph" else "stream", "plan": plan},
+        "us_per_call": round(us_per_step, 3),
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "algorithmic_bytes_per_call": wl.bytes,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel_us_avg_events": round(kernel_us, 3)},
+    }
+    if not args.no_cpu:
+        chk = check_against_oracle(wl)
+        out["cpu_baseline"] = {
+            "value": round(chk["sample_bytes"] / chk["cpu_seconds"] / 1e9, 4), "unit": "GB/s", "cores": 1,
+            "kind": "port",
+            "sample": f"the whole workload ({chk['rows']} rows x {wl.k}), single-threaded HOST_CHECK loop, "
+                      f"mean of {chk['cpu_reps']} runs, {chk['cpu_seconds']:.3f} s each",
+            "us_per_call": round(chk["cpu_seconds"] * 1e6, 1)}
+        out["parity"] = {"max_abs_err": chk["max_abs_err"], "max_rel_err": chk["max_rel_err"],
+                         "rel_floor": chk["rel_floor"], "tolerance_rel": 2e-3,
+                         "ok": bool(chk["max_rel_err"] <= 2e-3)}
+    others = {}
+    for name in [n for n in args.extra.split(",") if n and n != args.workload]:
+        w2 = Workload(name, device)
+        wall2, ev2, st2 = time_workload(w2, max(200, args.steps // 8), max(20, args.warmup // 4), use_graph=(args.launch == "graph"))
+        others[name] = {"workload": w2.description, "us_per_call": round(wall2 * 1e6 / st2, 3),
+                        "value_GBps": round(w2.bytes / (wall2 / st2) / 1e9, 1),
+                        "kernel_us_avg_events": round(ev2, 3),
+                        "roofline_frac": round(w2.bytes / (ev2 * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                        "buffer_sets_rotated": w2.sets, "steps": st2}
+        del w2
+        torch.cuda.empty_cache()
+    if others:
+        out["other_workloads"] = others
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -61,13 +61,23 @@ __device__ __forceinline__ int group_of(const GemvParams& p, int k_index) {
   return g < p.num_groups ? g : p.num_groups - 1;
 }
 
-// Everything one lane needs for one unit.
+// Everything one lane needs for one unit.  Scale and additive zero are kept as packed
+// (s, s) / (z, z) pairs in 32-bit registers.
 template <int BITS, int MB, int GROUPS_PER_RUN>
 struct UnitFragment {
-  u32x4 w[kBlocksPerUnit];                       // 4 chunks of this lane's row
-  uint32_t x[MB][BITS == 4 ? 4 : 2];             // this lane's piece of the activation run
-  half_t s[GROUPS_PER_RUN], z[GROUPS_PER_RUN];   // scale / additive zero of the run
+  u32x4 w[kBlocksPerUnit];                // 4 chunks of this lane's row
+  uint32_t x[MB][BITS == 4 ? 4 : 2];      // this lane's piece of the activation run
+  uint32_t s[GROUPS_PER_RUN];             // fp16 scale of each group of the run (low 16 bits)
+  uint32_t z[GROUPS_PER_RUN];             // fp16 additive zero (low 16 bits)
 };
+
+__device__ __forceinline__ uint32_t load_half_bits(const half_t* p) {
+  return (uint32_t)*reinterpret_cast<const uint16_t*>(p);
+}
+__device__ __forceinline__ half2_t splat_low(uint32_t bits) {
+  const half_t h = __builtin_bit_cast(half_t, (uint16_t)bits);
+  return half2_t{h, h};
+}
 
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f, const GemvParams& p,
@@ -94,54 +104,49 @@ __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>
     for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
       const int grp = group_of(p, k_run + gi * (G::kRunK / GROUPS_PER_RUN));
       const int idx = grp * p.n_out + row;
-      f.s[gi] = p.scale[idx];
-      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS) f.z[gi] = p.zero_add[idx];
+      f.s[gi] = load_half_bits(p.scale + idx);
+      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS) f.z[gi] = load_half_bits(p.zero_add + idx);
     }
+  }
+}
+
+// One 32-bit word of block I: convert, dequantise, dot.  Lane (4 I + J) of the DPP row holds
+// the activations that pair with this word.
+template <int BITS, bool HAS_ZERO, int MB, int I, int J>
+__device__ __forceinline__ void compute_word(float (&acc)[MB], uint32_t w, const uint32_t (&x)[MB][BITS == 4 ? 4 : 2],
+                                             const ConvertRegs& c, half2_t s2, half2_t z2) {
+  constexpr int kPairs = BITS == 4 ? 4 : 2;
+  half2_t q[kPairs];
+  if constexpr (BITS == 4) convert_int4_word(w, c, q); else convert_int8_word(w, c, q);
+#pragma unroll
+  for (int h = 0; h < kPairs; ++h) {
+    const half2_t d = dequant_pair<HAS_ZERO>(q[h], s2, z2);
+#pragma unroll
+    for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + J>(acc[m], x[m][h], d);
   }
 }
 
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, int I>
 __device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
-                                              const ConvertRegs& c, half_t col_scale) {
+                                              const ConvertRegs& c, half2_t col_scale2) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
   constexpr int gi = I * GROUPS_PER_RUN / kBlocksPerUnit;
-  const half2_t s2 = splat(QOP == MGEMV_PER_COLUMN_SCALE_ONLY ? col_scale : f.s[gi]);
-  const half2_t z2 = kHasZero ? splat(f.z[gi]) : half2_t{};
-  auto word = [&](auto J) {
-    constexpr int j = decltype(J)::value;
-    if constexpr (BITS == 4) {
-      half2_t q[4];
-      convert_int4_word(f.w[I][j], c, q);
-#pragma unroll
-      for (int h = 0; h < 4; ++h) {
-        const half2_t d = dequant_pair<kHasZero>(q[h], s2, z2);
-#pragma unroll
-        for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + j>(acc[m], f.x[m][h], d);
-      }
-    } else {
-      half2_t q[2];
-      convert_int8_word(f.w[I][j], c, q);
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const half2_t d = dequant_pair<kHasZero>(q[h], s2, z2);
-#pragma unroll
-        for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + j>(acc[m], f.x[m][h], d);
-      }
-    }
-  };
-  word(std::integral_constant<int, 0>{});
-  word(std::integral_constant<int, 1>{});
-  word(std::integral_constant<int, 2>{});
-  word(std::integral_constant<int, 3>{});
+  half2_t s2 = col_scale2, z2 = half2_t{};
+  if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) s2 = splat_low(f.s[gi]);
+  if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
+  compute_word<BITS, kHasZero, MB, I, 0>(acc, f.w[I][0], f.x, c, s2, z2);
+  compute_word<BITS, kHasZero, MB, I, 1>(acc, f.w[I][1], f.x, c, s2, z2);
+  compute_word<BITS, kHasZero, MB, I, 2>(acc, f.w[I][2], f.x, c, s2, z2);
+  compute_word<BITS, kHasZero, MB, I, 3>(acc, f.w[I][3], f.x, c, s2, z2);
 }
 
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
-                                             const ConvertRegs& c, half_t col_scale) {
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 0>(acc, f, c, col_scale);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 1>(acc, f, c, col_scale);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 2>(acc, f, c, col_scale);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 3>(acc, f, c, col_scale);
+                                             const ConvertRegs& c, half2_t col_scale2) {
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 0>(acc, f, c, col_scale2);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 1>(acc, f, c, col_scale2);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 2>(acc, f, c, col_scale2);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 3>(acc, f, c, col_scale2);
 }
 
 // blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: tiles_per_wg * split_k * MB * 64 floats.
@@ -183,13 +188,21 @@ gemv_dpp_kernel(const GemvParams p0) {
     __amdgpu_buffer_rsrc_t x_rsrc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) x_rsrc[m] = make_rsrc(p.x + (size_t)m * (size_t)p.k, (uint32_t)p.k * 2u);
-    half_t col_scale = (half_t)0.0f;
-    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = p.scale[row];
+    half2_t col_scale = half2_t{};
+    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = splat(p.scale[row]);
 
-    for (int u = 0; u < units; ++u) {
-      UnitFragment<BITS, MB, GROUPS_PER_RUN> f;
-      load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(f, p, w_rsrc, x_rsrc, u, ks_begin + u, lane, row);
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, f, c, col_scale);
+    // Two fragments in flight: the loads of unit u+1 are issued before unit u is computed, so
+    // a wave that is waiting for its turn on the VALU still has memory requests outstanding.
+    UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
+    load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, 0, ks_begin, lane, row);
+    int u = 0;
+    while (true) {
+      if (u + 1 < units) load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, u + 1, ks_begin + u + 1, lane, row);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale);
+      if (++u >= units) break;
+      if (u + 1 < units) load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, u + 1, ks_begin + u + 1, lane, row);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, col_scale);
+      if (++u >= units) break;
     }
 #pragma unroll
     for (int m = 0; m < MB; ++m) settle_dot_chain(acc[m]);
@@ -360,18 +373,25 @@ int groups_per_run(int group_size, int bits) {
   return 4;
 }
 
+// Launches through hipLaunchKernel so that the status returned is this launch's own, not a
+// stale sticky error left behind by some other runtime call of the process.
+template <typename Kernel, typename... Args>
+hipError_t launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+  void* argv[] = {static_cast<void*>(&args)...};
+  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream);
+}
+
 template <int BITS, int QOP, int MB>
 hipError_t launch_gemv_gpr(const GemvParams& p, int gpr, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
   if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
-    gemv_dpp_kernel<BITS, QOP, MB, 1><<<grid, block, lds, stream>>>(p);
+    return launch(gemv_dpp_kernel<BITS, QOP, MB, 1>, grid, block, lds, stream, p);
   } else {
     switch (gpr) {
-      case 1: gemv_dpp_kernel<BITS, QOP, MB, 1><<<grid, block, lds, stream>>>(p); break;
-      case 2: gemv_dpp_kernel<BITS, QOP, MB, 2><<<grid, block, lds, stream>>>(p); break;
-      default: gemv_dpp_kernel<BITS, QOP, MB, 4><<<grid, block, lds, stream>>>(p); break;
+      case 1: return launch(gemv_dpp_kernel<BITS, QOP, MB, 1>, grid, block, lds, stream, p);
+      case 2: return launch(gemv_dpp_kernel<BITS, QOP, MB, 2>, grid, block, lds, stream, p);
+      default: return launch(gemv_dpp_kernel<BITS, QOP, MB, 4>, grid, block, lds, stream, p);
     }
   }
-  return hipGetLastError();
 }
 
 template <int BITS, int QOP>
@@ -405,11 +425,10 @@ hipError_t launch_dequant(const GemvParams& p, int qop, half_t* out, hipStream_t
   const long long units = (long long)p.tiles * p.ksteps;
   const dim3 block(256), grid((unsigned)((units + 3) / 4));
   switch (qop) {
-    case 1: dequantize_kernel<BITS, 1><<<grid, block, 0, stream>>>(p, out); break;
-    case 2: dequantize_kernel<BITS, 2><<<grid, block, 0, stream>>>(p, out); break;
-    default: dequantize_kernel<BITS, 3><<<grid, block, 0, stream>>>(p, out); break;
+    case 1: return launch(dequantize_kernel<BITS, 1>, grid, block, 0, stream, p, out);
+    case 2: return launch(dequantize_kernel<BITS, 2>, grid, block, 0, stream, p, out);
+    default: return launch(dequantize_kernel<BITS, 3>, grid, block, 0, stream, p, out);
   }
-  return hipGetLastError();
 }
 
 }  // namespace mgemv
