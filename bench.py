@@ -121,19 +121,21 @@ def time_workload(wl, steps, warmup, use_graph=False):
     torch.cuda.synchronize()
     graph = None
     if use_graph:
-        # one rotation of the buffer sets captured once, replayed; launches only, no memsets
+        # whole rotations of the buffer sets (at least 32 kernel nodes, so that the cost of starting
+        # a replay is spread thin) captured once, replayed; launches only, no memsets
+        nodes = wl.sets * max(1, -(-32 // wl.sets))
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(side):
             with torch.cuda.graph(graph, stream=side):
-                for i in range(wl.sets):
+                for i in range(nodes):
                     wl.launch(i)
         torch.cuda.current_stream().wait_stream(side)
         graph.replay()
         torch.cuda.synchronize()
-        replays = max(1, steps // wl.sets)
-        steps = replays * wl.sets
+        replays = max(1, steps // nodes)
+        steps = replays * nodes
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -180,7 +182,7 @@ def check_against_oracle(wl, rows=None):
     got = wl.y.cpu().numpy()[:, :rows].astype(np.float64)
     r = ref.astype(np.float64)
     rms = float(np.sqrt(np.mean(r * r)))
-    floor = max(rms * 2.0 ** -10, 2.0 ** -24)
+    floor = max(rms * 2.0 ** -7, 2.0 ** -24)  # see tests/helpers.py:error_report for why 2^-7 * rms
     abs_err = np.abs(got - r)
     rel_err = abs_err / np.maximum(np.abs(r), floor)
     sample_bytes = algorithmic_bytes(rows, wl.k, wl.bits, wl.quant_op, wl.group, wl.m_batch, wl.has_bias)

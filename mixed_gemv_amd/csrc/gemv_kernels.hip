@@ -25,40 +25,53 @@ constexpr int kMaxWavesPerWorkgroup = 16;
 constexpr int kNumXcd = 8;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 
-struct GemvParams {
+// Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are the
+// ones a wave needs before it can issue its first loads; the build asks the compiler to
+// preload them into SGPRs at wave launch, which takes the kernarg fetch (a round trip to
+// memory) off the critical path of these microsecond-scale kernels.  Everything else sits in
+// GemvTail and is only needed once the k loop is under way.
+struct GemvTail {
+  const half_t* bias;
+  half_t* y;
+  int split_k;         // waves of a workgroup that share one tile (blockDim.x / 64)
+  int reserved;
+  long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
+};
+
+// Scalar view of one problem inside a kernel.
+struct Problem {
   const uint8_t* weights;
   const half_t* x;
   const half_t* scale;
   const half_t* zero_add;
-  const half_t* bias;
-  half_t* y;
   int n_out;
   int k;
-  int group_size;
-  int group_shift;     // log2(group_size) when it is a power of two, else -1
-  int num_groups;      // k / group_size (1 in per-column mode)
-  int tiles;           // ceil(n_out / 16)
   int ksteps;          // ceil(k / kStepK)
-  int split_k;         // waves of a workgroup that share one tile       (blockDim.x / 64)
-  int tiles_per_wg;    //                                                  (blockDim.y)
   int steps_per_wave;  // units per wave
-  int workgroups;      // logical workgroups per problem = ceil(tiles / tiles_per_wg)
+  int workgroups;      // logical workgroups = ceil(tiles / tiles_per_wg)
   int wgs_per_xcd;     // ceil(workgroups / 8); gridDim.x = 8 * wgs_per_xcd
-  long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
+  int group_size;
+  int tiles_per_wg;    // blockDim.y
 };
+
+constexpr uint32_t pack_steps(int ksteps, int steps_per_wave) { return (uint32_t)ksteps | ((uint32_t)steps_per_wave << 16); }
+constexpr uint32_t pack_group(int group_size, int tiles_per_wg) { return (uint32_t)group_size | ((uint32_t)tiles_per_wg << 24); }
 
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Neighbouring tiles read
 // neighbouring 32-byte pieces of the same scale/zero cache lines, so give each XCD (and its
 // private L2) a contiguous range of tiles instead of every eighth one.
-__device__ __forceinline__ int logical_workgroup(const GemvParams& p) {
+__device__ __forceinline__ int logical_workgroup(const Problem& p) {
   const int xcd = blockIdx.x % kNumXcd;
   const int slot = blockIdx.x / kNumXcd;
   return xcd * p.wgs_per_xcd + slot;
 }
 
-__device__ __forceinline__ int group_of(const GemvParams& p, int k_index) {
-  int g = p.group_shift >= 0 ? (k_index >> p.group_shift) : (k_index / p.group_size);
-  return g < p.num_groups ? g : p.num_groups - 1;
+// Group index of reduction position k_index (host/mixed_gemv.h:88), clamped to the last
+// group for the padded positions past k.
+__device__ __forceinline__ int group_of(const Problem& p, int k_index) {
+  k_index = k_index < p.k ? k_index : p.k - 1;
+  const bool pow2 = (p.group_size & (p.group_size - 1)) == 0;
+  return pow2 ? (k_index >> __builtin_ctz((unsigned)p.group_size)) : (k_index / p.group_size);
 }
 
 // Everything one lane needs for one unit.  Scale and additive zero are kept as packed
@@ -80,7 +93,7 @@ __device__ __forceinline__ half2_t splat_low(uint32_t bits) {
 }
 
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
-__device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f, const GemvParams& p,
+__device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f, const Problem& p,
                                           __amdgpu_buffer_rsrc_t w_rsrc, const __amdgpu_buffer_rsrc_t (&x_rsrc)[MB],
                                           int unit_in_wave, int kstep, int lane, int row) {
   using G = Geometry<BITS>;
@@ -149,19 +162,61 @@ __device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragmen
   compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 3>(acc, f, c, col_scale2);
 }
 
-// blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: tiles_per_wg * split_k * MB * 64 floats.
+// Sum over the four k slices of a wave: lanes l, l+16, l+32, l+48 hold the same row.
+// The result is valid in lanes 0..15.
+__device__ __forceinline__ float reduce_k_slices(float v) {
+  v += __shfl_down(v, 32);
+  v += __shfl_down(v, 16);
+  return v;
+}
+
+// Epilogue: fp32 add of the bias, one rounding to fp16
+// (host/mixed_gemv.h:102-103; epilogue/threadblock/epilogue.h:50-75).
+__device__ __forceinline__ void store_outputs(const GemvTail& tail, bool has_bias, int n_out, int m, int tile, int lane,
+                                              float sum) {
+  const int n = tile * kTileRows + lane;
+  if (lane < kTileRows && n < n_out) {
+    if (has_bias) sum += (float)tail.bias[n];
+    tail.y[(size_t)m * (size_t)n_out + n] = (half_t)sum;
+  }
+}
+
+// blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: tiles_per_wg * split_k * MB * 64 floats
+// (none when split_k == 1).
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __global__ void __launch_bounds__(kWave * kMaxWavesPerWorkgroup)
-gemv_dpp_kernel(const GemvParams p0) {
+gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
+                uint32_t packed_steps, int workgroups, int wgs_per_xcd, uint32_t packed_group, GemvTail tail) {
   extern __shared__ float partials[];
-  GemvParams p = p0;
-  const int batch = blockIdx.z;
-  p.weights += batch * p.stride_weights;
-  p.x += batch * p.stride_x;
-  p.scale += batch * p.stride_scale;
-  if (p.zero_add) p.zero_add += batch * p.stride_scale;
-  if (p.bias) p.bias += batch * p.stride_bias;
-  p.y += batch * p.stride_y;
+  Problem p;
+  p.weights = weights;
+  p.x = x;
+  p.scale = scale;
+  p.zero_add = zero_add;
+  p.n_out = n_out;
+  p.k = k;
+  p.ksteps = (int)(packed_steps & 0xffffu);
+  p.steps_per_wave = (int)(packed_steps >> 16);
+  p.workgroups = workgroups;
+  p.wgs_per_xcd = wgs_per_xcd;
+  p.group_size = (int)(packed_group & 0xffffffu);
+  p.tiles_per_wg = (int)(packed_group >> 24);
+  // Bring every kernel argument into SGPRs with ONE round trip to memory.  Left alone, the
+  // compiler sinks each scalar load next to its first use, which puts three or four dependent
+  // load-wait pairs in front of the first weight load of these microsecond-scale kernels.
+  asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
+               "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
+               "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale), "s"(tail.stride_bias),
+               "s"(tail.stride_y));
+  // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223); branch-free.
+  const long long batch = blockIdx.z;
+  p.weights += batch * tail.stride_weights;
+  p.x += batch * tail.stride_x;
+  p.scale += batch * tail.stride_scale;
+  p.zero_add += batch * tail.stride_scale;  // only dereferenced in scale+zero mode
+  const bool has_bias = tail.bias != nullptr;
+  tail.bias += batch * tail.stride_bias;
+  tail.y += batch * tail.stride_y;
 
   const int wg = logical_workgroup(p);
   if (wg >= p.workgroups) return;  // whole workgroup leaves before any barrier
@@ -170,6 +225,7 @@ gemv_dpp_kernel(const GemvParams p0) {
   const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // position along k
   const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);         // tile within the workgroup
   const int tile = wg * p.tiles_per_wg + ty;
+  const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
   const int row_raw = tile * kTileRows + lane % kTileRows;
   const int row = row_raw < p.n_out ? row_raw : p.n_out - 1;  // clamp padded rows (never stored)
 
@@ -179,8 +235,7 @@ gemv_dpp_kernel(const GemvParams p0) {
 
   const int ks_begin = kw * p.steps_per_wave;
   const int ks_end = min(ks_begin + p.steps_per_wave, p.ksteps);
-  if (tile < p.tiles && ks_begin < ks_end) {
-    const ConvertRegs c = make_convert_regs();
+  if (tile < tiles && ks_begin < ks_end) {
     const int units = ks_end - ks_begin;
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
         p.weights + ((size_t)tile * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
@@ -188,13 +243,14 @@ gemv_dpp_kernel(const GemvParams p0) {
     __amdgpu_buffer_rsrc_t x_rsrc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) x_rsrc[m] = make_rsrc(p.x + (size_t)m * (size_t)p.k, (uint32_t)p.k * 2u);
-    half2_t col_scale = half2_t{};
-    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = splat(p.scale[row]);
 
     // Two fragments in flight: the loads of unit u+1 are issued before unit u is computed, so
     // a wave that is waiting for its turn on the VALU still has memory requests outstanding.
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
     load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, 0, ks_begin, lane, row);
+    half2_t col_scale = half2_t{};
+    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = splat(p.scale[row]);
+    const ConvertRegs c = make_convert_regs();
     int u = 0;
     while (true) {
       if (u + 1 < units) load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, u + 1, ks_begin + u + 1, lane, row);
@@ -208,37 +264,48 @@ gemv_dpp_kernel(const GemvParams p0) {
     for (int m = 0; m < MB; ++m) settle_dot_chain(acc[m]);
   }
 
-  // Split-K / k-slice combine through LDS, fixed summation order.
-  const int slot = (ty * p.split_k + kw) * MB;
+  const int split_k = tail.split_k;
+  if (split_k == 1) {
+    // One wave owns the whole reduction of its tile: no LDS, no barrier.
+    if (tile < tiles) {
+#pragma unroll
+      for (int m = 0; m < MB; ++m) store_outputs(tail, has_bias, p.n_out, m, tile, lane, reduce_k_slices(acc[m]));
+    }
+    return;
+  }
+
+  // Split-K combine (gemv/threadblock/accumulator_combine.h:269-329): every wave parks its 64
+  // per-lane partial sums in LDS; after one barrier, wave kw of each tile sums activation rows
+  // m = kw, kw + split_k, ... over the waves in ascending order, then over the four k slices.
+  const int slot = (ty * split_k + kw) * MB;
 #pragma unroll
   for (int m = 0; m < MB; ++m) partials[(slot + m) * kWave + lane] = acc[m];
   __syncthreads();
-
-  const int tid = threadIdx.y * blockDim.x + threadIdx.x;
-  const int nthreads = blockDim.x * blockDim.y;
-  const int outputs = p.tiles_per_wg * MB * kTileRows;
-  for (int o = tid; o < outputs; o += nthreads) {
-    const int r = o % kTileRows;
-    const int m = (o / kTileRows) % MB;
-    const int t = o / (kTileRows * MB);
-    const int n = (wg * p.tiles_per_wg + t) * kTileRows + r;
-    if (n >= p.n_out) continue;
+  if (tile >= tiles) return;
+  for (int m = kw; m < MB; m += split_k) {
+    const float* part = partials + (ty * split_k * MB + m) * kWave + lane;
     float sum = 0.0f;
-    for (int w = 0; w < p.split_k; ++w) {
-      const float* part = partials + ((t * p.split_k + w) * MB + m) * kWave;
-#pragma unroll
-      for (int slice = 0; slice < kKSlices; ++slice) sum += part[slice * kTileRows + r];
+    int w = 0;
+    for (; w + 4 <= split_k; w += 4) {
+      const float a0 = part[(w + 0) * MB * kWave], a1 = part[(w + 1) * MB * kWave];
+      const float a2 = part[(w + 2) * MB * kWave], a3 = part[(w + 3) * MB * kWave];
+      sum = (((sum + a0) + a1) + a2) + a3;
     }
-    // Epilogue: fp32 add of the bias, one rounding to fp16
-    // (host/mixed_gemv.h:102-103; epilogue/threadblock/epilogue.h:50-75).
-    if (p.bias) sum += (float)p.bias[n];
-    p.y[(size_t)m * (size_t)p.n_out + n] = (half_t)sum;
+    for (; w < split_k; ++w) sum += part[w * MB * kWave];
+    store_outputs(tail, has_bias, p.n_out, m, tile, lane, reduce_k_slices(sum));
   }
 }
 
+struct DequantParams {
+  const uint8_t* weights;
+  const half_t* scale;
+  const half_t* zero_add;
+  int n_out, k, group_size, tiles, ksteps;
+};
+
 // One wave per unit; writes the dequantised weights of its 16 rows x kStepK columns.
 template <int BITS, int QOP>
-__global__ void __launch_bounds__(256) dequantize_kernel(const GemvParams p, half_t* __restrict__ out) {
+__global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, half_t* __restrict__ out) {
   using G = Geometry<BITS>;
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
   const int lane = threadIdx.x % kWave;
@@ -258,7 +325,10 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const GemvParams p, hal
     if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
       s = p.scale[row_c];
     } else {
-      const int idx = group_of(p, k0) * p.n_out + row_c;
+      Problem geo{};
+      geo.k = p.k;
+      geo.group_size = p.group_size;
+      const int idx = group_of(geo, k0) * p.n_out + row_c;
       s = p.scale[idx];
       if constexpr (kHasZero) z = p.zero_add[idx];
     }
@@ -299,20 +369,20 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 LaunchPlan plan_launch(int n_out, int k, int bits) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
-  // Aim for ~16 waves on each of the 256 compute units; a tile with few k steps cannot be
-  // split further than one unit per wave, and a workgroup holds at most 16 waves.
-  constexpr int kTargetWaves = 256 * 16;
-  int split_k = ceil_div(kTargetWaves, tiles);
+  // Measured on MI355X: one tile per workgroup and as many k-split waves as the tile has
+  // units (at most 16) is best or within a few percent of best for every shape tried, until
+  // the launch exceeds ~16k waves; beyond that halve the split so each wave keeps >= 2 units.
+  constexpr int kWaveBudget = 16384;
+  int split_k = ksteps < kMaxWavesPerWorkgroup ? ksteps : kMaxWavesPerWorkgroup;
+  while (split_k > 1 && (long long)tiles * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
+  int tiles_per_wg = 1;
   const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
   if (ov_sk > 0) split_k = ov_sk;
-  split_k = split_k < 1 ? 1 : split_k;
+  if (ov_tw > 0) tiles_per_wg = ov_tw;
   split_k = split_k > kMaxWavesPerWorkgroup ? kMaxWavesPerWorkgroup : split_k;
   split_k = split_k > ksteps ? ksteps : split_k;
   const int steps = ceil_div(ksteps, split_k);
   split_k = ceil_div(ksteps, steps);
-  int tiles_per_wg = 4 / split_k;  // keep workgroups at >= 256 threads where the split allows
-  if (ov_tw > 0) tiles_per_wg = ov_tw;
-  if (tiles_per_wg < 1) tiles_per_wg = 1;
   if (tiles_per_wg * split_k > kMaxWavesPerWorkgroup) tiles_per_wg = kMaxWavesPerWorkgroup / split_k;
   LaunchPlan lp;
   lp.split_k = split_k;
@@ -344,26 +414,11 @@ int check_problem(const void* weights, const void* scale, const void* zero_add, 
   // 32-bit index arithmetic inside the kernels
   const long long groups = k / group_size;
   if (groups * (long long)n_out >= (1ll << 30)) return MGEMV_ERR_SIZE;
-  if ((long long)num_ksteps(k, weight_bits) * kUnitBytes >= (1ll << 31)) return MGEMV_ERR_SIZE;
+  if (num_ksteps(k, weight_bits) > 0xffff || group_size >= (1 << 24)) return MGEMV_ERR_SIZE;
   if ((long long)k * 2 * MGEMV_MAX_M_BATCH >= (1ll << 31)) return MGEMV_ERR_SIZE;
   if (reinterpret_cast<uintptr_t>(weights) % 16) return MGEMV_ERR_ALIGNMENT;
   if (reinterpret_cast<uintptr_t>(scale) % 2 || reinterpret_cast<uintptr_t>(zero_add) % 2) return MGEMV_ERR_ALIGNMENT;
   return MGEMV_OK;
-}
-
-void fill_common(GemvParams& p, const void* weights, const uint16_t* scale, const uint16_t* zero_add, int n_out,
-                 int k, int group_size, int quant_op, int weight_bits) {
-  p = GemvParams{};
-  p.weights = static_cast<const uint8_t*>(weights);
-  p.scale = reinterpret_cast<const half_t*>(scale);
-  p.zero_add = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? reinterpret_cast<const half_t*>(zero_add) : nullptr;
-  p.n_out = n_out;
-  p.k = k;
-  p.group_size = group_size;
-  p.group_shift = (group_size & (group_size - 1)) == 0 ? __builtin_ctz((unsigned)group_size) : -1;
-  p.num_groups = k / group_size;
-  p.tiles = num_tiles(n_out);
-  p.ksteps = num_ksteps(k, weight_bits);
 }
 
 int groups_per_run(int group_size, int bits) {
@@ -381,47 +436,67 @@ hipError_t launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t 
   return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream);
 }
 
+// Host-side description of one GEMV launch.
+struct GemvLaunch {
+  const uint8_t* weights;
+  const half_t* x;
+  const half_t* scale;
+  const half_t* zero_add;
+  int n_out, k, group_size;
+  LaunchPlan plan;
+  GemvTail tail;
+  dim3 grid, block;
+  size_t lds;
+  hipStream_t stream;
+};
+
+template <int BITS, int QOP, int MB, int GPR>
+hipError_t launch_gemv_kernel(const GemvLaunch& g) {
+  return launch(gemv_dpp_kernel<BITS, QOP, MB, GPR>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
+                g.zero_add, g.n_out, g.k, pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups,
+                g.plan.wgs_per_xcd, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+}
+
 template <int BITS, int QOP, int MB>
-hipError_t launch_gemv_gpr(const GemvParams& p, int gpr, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+hipError_t launch_gemv_gpr(const GemvLaunch& g, int gpr) {
   if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
-    return launch(gemv_dpp_kernel<BITS, QOP, MB, 1>, grid, block, lds, stream, p);
+    return launch_gemv_kernel<BITS, QOP, MB, 1>(g);
   } else {
     switch (gpr) {
-      case 1: return launch(gemv_dpp_kernel<BITS, QOP, MB, 1>, grid, block, lds, stream, p);
-      case 2: return launch(gemv_dpp_kernel<BITS, QOP, MB, 2>, grid, block, lds, stream, p);
-      default: return launch(gemv_dpp_kernel<BITS, QOP, MB, 4>, grid, block, lds, stream, p);
+      case 1: return launch_gemv_kernel<BITS, QOP, MB, 1>(g);
+      case 2: return launch_gemv_kernel<BITS, QOP, MB, 2>(g);
+      default: return launch_gemv_kernel<BITS, QOP, MB, 4>(g);
     }
   }
 }
 
 template <int BITS, int QOP>
-hipError_t launch_gemv_mb(const GemvParams& p, int mb, int gpr, dim3 grid, dim3 block, size_t lds, hipStream_t stream) {
+hipError_t launch_gemv_mb(const GemvLaunch& g, int mb, int gpr) {
   switch (mb) {
-    case 1: return launch_gemv_gpr<BITS, QOP, 1>(p, gpr, grid, block, lds, stream);
-    case 2: return launch_gemv_gpr<BITS, QOP, 2>(p, gpr, grid, block, lds, stream);
-    case 3: return launch_gemv_gpr<BITS, QOP, 3>(p, gpr, grid, block, lds, stream);
-    default: return launch_gemv_gpr<BITS, QOP, 4>(p, gpr, grid, block, lds, stream);
+    case 1: return launch_gemv_gpr<BITS, QOP, 1>(g, gpr);
+    case 2: return launch_gemv_gpr<BITS, QOP, 2>(g, gpr);
+    case 3: return launch_gemv_gpr<BITS, QOP, 3>(g, gpr);
+    default: return launch_gemv_gpr<BITS, QOP, 4>(g, gpr);
   }
 }
 
-hipError_t launch_gemv(const GemvParams& p, int bits, int qop, int mb, int gpr, dim3 grid, dim3 block, size_t lds,
-                       hipStream_t stream) {
+hipError_t launch_gemv(const GemvLaunch& g, int bits, int qop, int mb, int gpr) {
   if (bits == 4) {
     switch (qop) {
-      case 1: return launch_gemv_mb<4, 1>(p, mb, gpr, grid, block, lds, stream);
-      case 2: return launch_gemv_mb<4, 2>(p, mb, gpr, grid, block, lds, stream);
-      default: return launch_gemv_mb<4, 3>(p, mb, gpr, grid, block, lds, stream);
+      case 1: return launch_gemv_mb<4, 1>(g, mb, gpr);
+      case 2: return launch_gemv_mb<4, 2>(g, mb, gpr);
+      default: return launch_gemv_mb<4, 3>(g, mb, gpr);
     }
   }
   switch (qop) {
-    case 1: return launch_gemv_mb<8, 1>(p, mb, gpr, grid, block, lds, stream);
-    case 2: return launch_gemv_mb<8, 2>(p, mb, gpr, grid, block, lds, stream);
-    default: return launch_gemv_mb<8, 3>(p, mb, gpr, grid, block, lds, stream);
+    case 1: return launch_gemv_mb<8, 1>(g, mb, gpr);
+    case 2: return launch_gemv_mb<8, 2>(g, mb, gpr);
+    default: return launch_gemv_mb<8, 3>(g, mb, gpr);
   }
 }
 
 template <int BITS>
-hipError_t launch_dequant(const GemvParams& p, int qop, half_t* out, hipStream_t stream) {
+hipError_t launch_dequant(const DequantParams& p, int qop, half_t* out, hipStream_t stream) {
   const long long units = (long long)p.tiles * p.ksteps;
   const dim3 block(256), grid((unsigned)((units + 3) / 4));
   switch (qop) {
@@ -449,34 +524,33 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
     return MGEMV_ERR_ALIGNMENT;
   if (stride_weights % 16 || stride_x % 8) return MGEMV_ERR_ALIGNMENT;
 
-  GemvParams p;
-  fill_common(p, weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits);
-  p.bias = reinterpret_cast<const half_t*>(bias);
-  p.stride_weights = stride_weights;
-  p.stride_x = stride_x;
-  p.stride_scale = stride_scale;
-  p.stride_bias = stride_bias;
-  p.stride_y = stride_y;
-  const LaunchPlan lp = plan_launch(n_out, k, weight_bits);
-  p.split_k = lp.split_k;
-  p.tiles_per_wg = lp.tiles_per_wg;
-  p.steps_per_wave = lp.steps_per_wave;
-  p.workgroups = lp.workgroups;
-  p.wgs_per_xcd = lp.wgs_per_xcd;
-  const dim3 grid((unsigned)(lp.wgs_per_xcd * kNumXcd), 1, (unsigned)batch_count);
-  const dim3 block((unsigned)(kWave * lp.split_k), (unsigned)lp.tiles_per_wg, 1);
+  GemvLaunch g{};
+  g.weights = static_cast<const uint8_t*>(weights);
+  g.scale = reinterpret_cast<const half_t*>(scale);
+  g.zero_add = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? reinterpret_cast<const half_t*>(zero_add) : nullptr;
+  g.n_out = n_out;
+  g.k = k;
+  g.group_size = group_size;
+  g.plan = plan_launch(n_out, k, weight_bits);
+  g.tail.bias = reinterpret_cast<const half_t*>(bias);
+  g.tail.split_k = g.plan.split_k;
+  g.tail.stride_weights = stride_weights;
+  g.tail.stride_x = stride_x;
+  g.tail.stride_scale = stride_scale;
+  g.tail.stride_bias = stride_bias;
+  g.tail.stride_y = stride_y;
+  g.grid = dim3((unsigned)(g.plan.wgs_per_xcd * kNumXcd), 1, (unsigned)batch_count);
+  g.block = dim3((unsigned)(kWave * g.plan.split_k), (unsigned)g.plan.tiles_per_wg, 1);
+  g.stream = static_cast<hipStream_t>(stream);
   const int gpr = groups_per_run(group_size, weight_bits);
 
   // Activation rows are processed kMaxValuBatch at a time.
   for (int m0 = 0; m0 < m_batch; m0 += kMaxValuBatch) {
     const int mb = m_batch - m0 < kMaxValuBatch ? m_batch - m0 : kMaxValuBatch;
-    GemvParams q = p;
-    q.x = reinterpret_cast<const half_t*>(x) + (size_t)m0 * (size_t)k;
-    q.y = reinterpret_cast<half_t*>(y) + (size_t)m0 * (size_t)n_out;
-    const size_t lds = (size_t)lp.tiles_per_wg * lp.split_k * mb * kWave * sizeof(float);
-    if (launch_gemv(q, weight_bits, quant_op, mb, gpr, grid, block, lds, static_cast<hipStream_t>(stream)) !=
-        hipSuccess)
-      return MGEMV_ERR_LAUNCH;
+    g.x = reinterpret_cast<const half_t*>(x) + (size_t)m0 * (size_t)k;
+    g.tail.y = reinterpret_cast<half_t*>(y) + (size_t)m0 * (size_t)n_out;
+    g.lds = g.plan.split_k == 1 ? 0 : (size_t)g.plan.tiles_per_wg * g.plan.split_k * mb * kWave * sizeof(float);
+    if (launch_gemv(g, weight_bits, quant_op, mb, gpr) != hipSuccess) return MGEMV_ERR_LAUNCH;
   }
   return MGEMV_OK;
 }
@@ -494,8 +568,15 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(out) % 4) return MGEMV_ERR_ALIGNMENT;
-  GemvParams p;
-  fill_common(p, weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits);
+  DequantParams p{};
+  p.weights = static_cast<const uint8_t*>(weights);
+  p.scale = reinterpret_cast<const half_t*>(scale);
+  p.zero_add = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? reinterpret_cast<const half_t*>(zero_add) : nullptr;
+  p.n_out = n_out;
+  p.k = k;
+  p.group_size = group_size;
+  p.tiles = num_tiles(n_out);
+  p.ksteps = num_ksteps(k, weight_bits);
   const hipError_t e = weight_bits == 4
                            ? launch_dequant<4>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream))
                            : launch_dequant<8>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream));

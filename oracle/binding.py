@@ -36,6 +36,9 @@ def lib():
             getattr(h, name).argtypes = [c.c_uint16, c.c_uint16]
         h.orc_h_fma.restype = c.c_uint16
         h.orc_h_fma.argtypes = [c.c_uint16] * 3
+        for name, nargs in (("orc_f16_to_f32_n", 2), ("orc_f32_to_f16_n", 2), ("orc_h_mul_n", 3), ("orc_h_add_n", 3),
+                            ("orc_h_fma_n", 4)):
+            getattr(h, name).argtypes = [vp] * nargs + [c.c_size_t]
         h.orc_pack_int4.argtypes = [vp, vp, c.c_size_t]
         h.orc_unpack_int4.argtypes = [vp, vp, c.c_size_t]
         h.orc_fold_zero_points.argtypes = [vp, vp, vp, c.c_size_t]
@@ -87,6 +90,46 @@ def h_add(a, b):
 
 def h_fma(a, b, c):
     return int(lib().orc_h_fma(int(a), int(b), int(c)))
+
+
+def f16_to_f32_array(bits):
+    b = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(b.shape, dtype=np.float32)
+    lib().orc_f16_to_f32_n(_p(out), _p(b), b.size)
+    return out
+
+
+def f32_to_f16_array(values):
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(v.shape, dtype=np.uint16)
+    lib().orc_f32_to_f16_n(_p(out), _p(v), v.size)
+    return out
+
+
+def _binary(fn, a, b):
+    a = np.ascontiguousarray(a, dtype=np.uint16)
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    assert a.shape == b.shape
+    out = np.empty(a.shape, dtype=np.uint16)
+    fn(_p(out), _p(a), _p(b), a.size)
+    return out
+
+
+def h_mul_array(a, b):
+    return _binary(lib().orc_h_mul_n, a, b)
+
+
+def h_add_array(a, b):
+    return _binary(lib().orc_h_add_n, a, b)
+
+
+def h_fma_array(a, b, c):
+    a = np.ascontiguousarray(a, dtype=np.uint16)
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    c = np.ascontiguousarray(c, dtype=np.uint16)
+    out = np.empty(a.shape, dtype=np.uint16)
+    lib().orc_h_fma_n(_p(out), _p(a), _p(b), _p(c), a.size)
+    return out
 
 
 # ---- host utilities ----------------------------------------------------------------------

@@ -174,6 +174,23 @@ ORC_API uint16_t orc_h_fma(uint16_t a, uint16_t b, uint16_t c) {
   return (uint16_t)(sign | out);
 }
 
+/* array forms of the scalar helpers, for vectorised checks in the tests */
+ORC_API void orc_f16_to_f32_n(float *out, const uint16_t *in, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = orc_f16_to_f32(in[i]);
+}
+ORC_API void orc_f32_to_f16_n(uint16_t *out, const float *in, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = orc_f32_to_f16(in[i]);
+}
+ORC_API void orc_h_mul_n(uint16_t *out, const uint16_t *a, const uint16_t *b, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = h_mul(a[i], b[i]);
+}
+ORC_API void orc_h_add_n(uint16_t *out, const uint16_t *a, const uint16_t *b, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = h_add(a[i], b[i]);
+}
+ORC_API void orc_h_fma_n(uint16_t *out, const uint16_t *a, const uint16_t *b, const uint16_t *c, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = orc_h_fma(a[i], b[i], c[i]);
+}
+
 /* ------------------------------------------------------------------------------------ */
 /* int4 packing: utils/preprocess.h:41-84, utils/vector_subbyte.h:55-67,150-156           */
 /* element 2i -> bits 0..3 of byte i, element 2i+1 -> bits 4..7                           */

@@ -52,12 +52,24 @@ class Problem:
                         self.group_size, self.quant_op, self.bits, threads=threads)
 
 
+REL_FLOOR_FRACTION = 2.0 ** -7
+
+
 def error_report(got, ref):
-    """max abs error, and max relative error with denominator max(|ref|, 2^-10 * rms(ref))."""
+    """max abs error, and max relative error with denominator max(|ref|, 2^-7 * rms(ref)).
+
+    Why a floor, and why this one: an output that happens to be almost zero is a sum of
+    thousands of cancelling terms, and its ABSOLUTE error is set by the order in which fp32
+    adds them (a few 1e-5 for k = 8192 with outputs of rms 3).  The reference's own ascending-k
+    HOST_CHECK loop differs from the exactly accumulated, once-rounded result by 2.8e-3
+    relative when the floor is 2^-10 * rms, i.e. it would fail a 2e-3 bar against the truth;
+    from 2^-7 * rms upwards its deviation is the half-ulp rounding level (9.7e-4), so that is
+    the smallest floor under which "within 2e-3 of HOST_CHECK" is a statement about the kernel
+    and not about summation order."""
     g = np.asarray(got, dtype=np.float64).reshape(-1)
     r = np.asarray(ref, dtype=np.float64).reshape(-1)
     rms = float(np.sqrt(np.mean(r * r))) if r.size else 0.0
-    floor = max(rms * 2.0 ** -10, 2.0 ** -24)
+    floor = max(rms * REL_FLOOR_FRACTION, 2.0 ** -24)
     abs_err = np.abs(g - r)
     rel = abs_err / np.maximum(np.abs(r), floor)
     return float(abs_err.max(initial=0.0)), float(rel.max(initial=0.0)), floor

@@ -1,0 +1,188 @@
+"""Host side of the library (no GPU needed): packing, zero folding, the gfx950 weight
+preprocessor, error codes, and that the shared library exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import mixed_gemv_amd as mg
+import oracle as orc
+from mixed_gemv_amd import _lib
+from mixed_gemv_amd._lib import MixedGemvError
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+W4, W8 = mg.QuantType.W4_A16, mg.QuantType.W8_A16
+COL, ROW = mg.LayoutType.kColumnMajor, mg.LayoutType.kRowMajor
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(REPO, "include", "mixed_gemv.h")).read()
+    declared = set(re.findall(r"MGEMV_API\s+[\w\s\*]+?\b(mgemv_\w+)\s*\(", header))
+    assert len(declared) >= 12
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(handle, name), f"{name} declared in include/mixed_gemv.h but not exported"
+    assert declared == set(_lib.SIGNATURES), "python binding and header disagree"
+    assert _lib.lib().mgemv_version() >= 100
+    for code in range(0, 14):
+        assert _lib.lib().mgemv_status_string(code)
+
+
+def test_pack_unpack_and_fold_equal_the_oracle():
+    q = orc.fill_int8(4096, 3, -8, 7)
+    packed = mg.SubBytePacker.pack(q)
+    assert np.array_equal(packed, orc.pack_int4(q))
+    assert np.array_equal(mg.SubBytePacker.unpack(packed), q)
+    every = np.arange(256, dtype=np.uint8)
+    assert np.array_equal(mg.SubBytePacker.unpack(every), orc.unpack_int4(every))
+    # all finite scales x a spread of zero points
+    bits = np.arange(65536, dtype=np.uint16)
+    finite = bits[(bits & 0x7C00) != 0x7C00]
+    for z in (-128, -8, -1, 0, 1, 7, 127):
+        zz = np.full(finite.shape, z, dtype=np.int8)
+        got = mg.ZeroPointPreprocessor.neg_zero_point_multiplies_scale(finite.view(np.float16), zz)
+        assert np.array_equal(got.view(np.uint16), orc.fold_zero_points(finite.view(np.float16), zz).view(np.uint16))
+
+
+def _expected_offset(n, k0, k, bits):
+    """Layout closed form restated independently of csrc/tile_layout.h."""
+    chunk = 128 // bits
+    run, step = 4 * chunk, 16 * chunk
+    ksteps = -(-k // step)
+    tile, r = divmod(n, 16)
+    s, kk = divmod(k0, step)
+    slice_, rem = divmod(kk, run)
+    blk = rem // chunk
+    return (tile * ksteps + s) * 4096 + blk * 1024 + (slice_ * 16 + r) * 16
+
+
+@pytest.mark.parametrize("bits,n_out,k", [(4, 16, 512), (4, 20, 544), (4, 100, 1120), (8, 16, 256), (8, 36, 400)])
+def test_preprocess_layout_closed_form_and_round_trip(bits, n_out, k):
+    lo, hi = (-8, 7) if bits == 4 else (-128, 127)
+    q = orc.fill_int8(n_out * k, 100 + n_out, lo, hi).reshape(n_out, k)
+    raw = orc.pack_int4(q.reshape(-1)) if bits == 4 else q.reshape(-1).view(np.uint8)
+    qt = W4 if bits == 4 else W8
+    pre = mg.MixedGemvWeightPreprocessor.run(raw, (k, n_out), COL, qt)
+    assert pre.size == mg.preprocessed_size((k, n_out), qt)
+    assert pre.size == -(-n_out // 16) * -(-k // (2048 // bits)) * 4096
+    chunk = 128 // bits
+    touched = np.zeros(pre.size, dtype=bool)
+    for n in range(n_out):
+        for k0 in range(0, k, chunk):
+            off = _expected_offset(n, k0, k, bits)
+            words = pre[off:off + 16].view(np.uint32)
+            touched[off:off + 16] = True
+            vals = q[n, k0:k0 + chunk].astype(np.int32)
+            for j in range(4):
+                w = int(words[j])
+                if bits == 4:
+                    for e in range(8):
+                        pos = (e % 2) * 4 + e // 2           # pair (e, e+1) sits in the two 16-bit halves
+                        assert ((w >> (4 * pos)) & 0xF) == vals[8 * j + e] + 8
+                else:
+                    for e in range(4):
+                        assert ((w >> (8 * e)) & 0xFF) == vals[4 * j + e] + 128
+    assert not pre[~touched].any(), "padding must be zero"
+    back = mg.unpreprocess_weights(pre, (k, n_out), qt)
+    assert np.array_equal(back, raw)
+
+
+def test_preprocess_is_a_bijection_on_nibbles():
+    n_out, k = 32, 1024
+    # every nibble distinct-ish: use a counter pattern so that a collision or a dropped chunk shows
+    raw = (np.arange(n_out * k // 2, dtype=np.uint32) * 2654435761 >> 7).astype(np.uint8)
+    pre = mg.MixedGemvWeightPreprocessor.run(raw, (k, n_out), COL, W4)
+    assert np.array_equal(np.sort(mg.SubBytePacker.unpack(pre)), np.sort(mg.SubBytePacker.unpack(raw ^ 0x88).astype(np.int8)))
+    assert np.array_equal(mg.unpreprocess_weights(pre, (k, n_out), W4), raw)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_row_major_input_equals_transposed_column_major(bits):
+    n_out, k = 48, 320
+    lo, hi = (-8, 7) if bits == 4 else (-128, 127)
+    q = orc.fill_int8(n_out * k, 55, lo, hi).reshape(n_out, k)          # [n_out][k]
+    qt = W4 if bits == 4 else W8
+    to_raw = (lambda a: orc.pack_int4(a.reshape(-1))) if bits == 4 else (lambda a: a.reshape(-1).view(np.uint8).copy())
+    col = mg.MixedGemvWeightPreprocessor.run(to_raw(q), (k, n_out), COL, qt)
+    row = mg.MixedGemvWeightPreprocessor.run(to_raw(np.ascontiguousarray(q.T)), (k, n_out), ROW, qt)
+    assert np.array_equal(col, row)
+
+
+def test_three_dimensional_shape_is_per_expert():
+    e, n_out, k = 3, 20, 96
+    q = orc.fill_int8(e * n_out * k, 66, -8, 7).reshape(e, n_out, k)
+    raw = orc.pack_int4(q.reshape(-1))
+    pre = mg.MixedGemvWeightPreprocessor.run(raw, (e, k, n_out), COL, W4)
+    one = mg.preprocessed_size((k, n_out), W4)
+    assert pre.size == e * one
+    for i in range(e):
+        single = mg.MixedGemvWeightPreprocessor.run(orc.pack_int4(q[i].reshape(-1)), (k, n_out), COL, W4)
+        assert np.array_equal(pre[i * one:(i + 1) * one], single)
+    assert np.array_equal(mg.unpreprocess_weights(pre, (e, k, n_out), W4), raw)
+
+
+def test_preprocess_error_codes():
+    buf = np.zeros(1 << 16, dtype=np.uint8)
+    cases = [
+        ((64,), COL, W4, 2),            # rank 1          utils/preprocess.h:486-489
+        ((1, 2, 64, 64), COL, W4, 2),   # rank 4
+        ((64, 6), COL, W4, 3),          # rows % 4        utils/preprocess.h:319-322
+        ((40, 64), COL, W4, 4),         # k % 32 (int4)   utils/preprocess.h:324-327
+        ((24, 64), COL, W8, 4),         # k % 16 (int8)
+        ((64, 64), COL, mg.QuantType.W4_AFP8, 7),
+        ((64, 64), 5, W4, 9),
+        ((0, 64), COL, W4, 10),
+    ]
+    for shape, layout, qt, status in cases:
+        with pytest.raises(MixedGemvError) as ei:
+            mg.MixedGemvWeightPreprocessor.run(buf, shape, layout, qt)
+        assert ei.value.status == status, (shape, ei.value.status)
+    assert mg.preprocessed_size((64,), W4) == 0
+    lib = _lib.lib()
+    shape = (ctypes.c_size_t * 2)(64, 64)
+    assert lib.mgemv_preprocess_weights(None, None, shape, 2, 1, 1) == 1
+    assert lib.mgemv_pack_int4(None, None, 8) == 1
+    assert lib.mgemv_pack_int4(None, None, 0) == 0
+    assert lib.mgemv_fold_zero_points(None, None, None, 4) == 1
+
+
+def test_gemv_argument_checks_return_codes_without_launching():
+    """Every condition on which the reference prints and exits is a status code here; all of
+    these return before anything touches a GPU."""
+    lib = _lib.lib()
+    p = ctypes.c_void_p(0x1000)  # never dereferenced: the checks below all fail first
+
+    def gemv(n_out=64, m=1, k=512, g=128, qop=3, bits=4, w=p, x=p, s=p, z=p, y=p):
+        return lib.mgemv_gemv(w, x, s, z, None, y, n_out, m, k, g, qop, bits, None)
+
+    assert gemv(qop=0) == 6 and gemv(qop=4) == 6          # gemv/weight_only_quant_op.h:12-18
+    assert gemv(bits=5) == 7
+    assert gemv(m=0) == 8 and gemv(m=17) == 8              # the reference accepts N == 1 only (host/mixed_gemv.h:72-75)
+    assert gemv(n_out=0) == 10 and gemv(k=-4) == 10
+    assert gemv(n_out=66) == 3
+    assert gemv(k=520) == 4
+    assert gemv(g=32) == 5                                  # gemv/device/gemv_adaptor.h:199-203
+    assert gemv(g=96, k=512) == 5                           # does not divide k
+    assert gemv(g=80, k=640) == 5                           # not a multiple of 32
+    assert gemv(w=None) == 1 and gemv(s=None) == 1 and gemv(z=None) == 1 and gemv(x=None) == 1 and gemv(y=None) == 1
+    assert gemv(w=ctypes.c_void_p(0x1008)) == 13
+    assert gemv(x=ctypes.c_void_p(0x1002)) == 13
+    assert lib.mgemv_gemv_batched(p, p, p, p, None, p, 0, 64, 1, 512, 128, 3, 4, 0, 0, 0, 0, 0, None) == 8
+    assert lib.mgemv_dequantize(p, p, p, None, 64, 512, 128, 3, 4, None) == 1
+    assert lib.mgemv_dequantize(p, p, p, p, 64, 512, 16, 2, 4, None) == 5
+    # per-column mode ignores group_size entirely (mixed_gemv_test.cu:142-143): 16 would be rejected otherwise
+    assert lib.mgemv_dequantize(p, p, None, None, 64, 512, 16, 1, 4, None) == 1
+    out = (ctypes.c_int * 6)()
+    assert lib.mgemv_query_launch(4096, 1, 4096, 4, ctypes.byref(out)) == 0
+    assert out[0] % 8 == 0 and out[1] % 64 == 0 and out[2] * out[4] >= 8
+    assert lib.mgemv_query_launch(4096, 1, 4096, 3, ctypes.byref(out)) == 7
+    assert lib.mgemv_set_launch_override(-1, 0) == 10
+
+
+def test_adaptor_mirror_rejects_small_groups_like_the_reference():
+    args = mg.GemvAdaptor.Arguments((64, 1, 512), 0x1000, 0x1000, 0x1000, 0x1000, None, 0x1000, group_size=32)
+    with pytest.raises(MixedGemvError) as ei:
+        mg.GemvAdaptor().initialize(args)
+    assert ei.value.status == 5
