@@ -162,14 +162,22 @@ MGEMV_API int mgemv_dequantize(const void *weights, const uint16_t *scale, const
                                uint16_t *out, int n_out, int k, int group_size, int quant_op, int weight_bits,
                                void *stream);
 
-/* Launch geometry override for tuning and tests: k-split waves per tile and tiles per
- * workgroup; 0 restores the built-in heuristic.  Process-wide. */
-MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup);
+/* Launch geometry override for tuning and tests: k-split waves per tile, tiles (tile groups)
+ * per workgroup, and tiles handled by one wave of the matrix-core kernel (1, 2 or 4); 0
+ * restores the built-in heuristic for that knob.  Process-wide.  These are the counterparts of
+ * the reference's compile-time ThreadBlockShape / WarpShape choices (mixed_gemv_test.cu:67-70). */
+MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave);
+
+/* Smallest m_batch served by the matrix-core kernel instead of the VALU kernel (built-in
+ * default 5; 0 restores it; 17 keeps every batch size on the VALU kernel).  For tuning and
+ * tests.  Process-wide. */
+MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Reports the geometry mgemv_gemv would use: out[0] = workgroups, out[1] = threads per
- * workgroup, out[2] = k-split waves per tile, out[3] = tiles per workgroup,
- * out[4] = wave steps per wave, out[5] = 1 when the matrix-core path is chosen. */
-MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[6]);
+ * workgroup, out[2] = k-split waves per tile, out[3] = tiles (tile groups) per workgroup,
+ * out[4] = wave steps per wave, out[5] = 1 when the matrix-core path is chosen,
+ * out[6] = tiles per wave. */
+MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[7]);
 
 #ifdef __cplusplus
 }

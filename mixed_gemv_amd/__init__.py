@@ -17,6 +17,7 @@ from .api import (  # noqa: F401
     preprocessed_size,
     query_launch,
     set_launch_override,
+    set_matrix_core_threshold,
     unpreprocess_weights,
 )
 from ._lib import LIB_PATH, MixedGemvError  # noqa: F401

@@ -207,13 +207,18 @@ def dequantize(ptr_A, ptr_scale, ptr_zero_point, ptr_out, M, K, group_size,
     _lib.check(st, "dequantize")
 
 
-def set_launch_override(split_k_waves=0, tiles_per_workgroup=0):
-    _lib.check(_lib.lib().mgemv_set_launch_override(int(split_k_waves), int(tiles_per_workgroup)), "set_launch_override")
+def set_launch_override(split_k_waves=0, tiles_per_workgroup=0, tiles_per_wave=0):
+    _lib.check(_lib.lib().mgemv_set_launch_override(int(split_k_waves), int(tiles_per_workgroup), int(tiles_per_wave)),
+               "set_launch_override")
+
+
+def set_matrix_core_threshold(min_m_batch=0):
+    _lib.check(_lib.lib().mgemv_set_matrix_core_threshold(int(min_m_batch)), "set_matrix_core_threshold")
 
 
 def query_launch(n_out, m_batch, k, weight_bits=4):
-    out = (ctypes.c_int * 6)()
+    out = (ctypes.c_int * 7)()
     _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), ctypes.byref(out)),
                "query_launch")
-    keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core")
+    keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave")
     return dict(zip(keys, list(out)))

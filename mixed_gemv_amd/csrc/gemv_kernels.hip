@@ -22,6 +22,7 @@ namespace mgemv {
 
 constexpr int kWave = 64;
 constexpr int kMaxWavesPerWorkgroup = 16;
+constexpr int kMaxWavesPerMfmaWorkgroup = 8;  // leaves each wave of the matrix-core kernel 256 VGPRs
 constexpr int kNumXcd = 8;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 
@@ -296,6 +297,246 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Small-batch variant on the matrix cores (5 <= m_batch <= 16, padded to 16 columns).
+//
+// The tile layout already has the operand shape of v_mfma_f32_16x16x32_f16: lane l holds
+// row l % 16 of the tile and k slice l / 16, and one 32-bit weight word dequantises to the 8
+// consecutive-k fp16 values (4 VGPRs) that lane contributes to the 16 x 32 weight operand.
+// The activation operand is read straight from x: lane l supplies x[l % 16][same 8 k].  The
+// instruction pairs operand elements of equal (k slice, element) position, so the result is
+// D[row][batch row] = sum_k dq[row][k] * x[batch row][k], accumulated in fp32 across the
+// wave's whole k range: the VALU only converts and dequantises (no dot instructions), which
+// is what makes this path faster than repeating the VALU kernel once activation rows multiply.
+// It replaces nothing in the reference, whose kernel is fixed to one activation row
+// (gemv/threadblock/default_mma_core_simt.h:68-70).
+// ---------------------------------------------------------------------------------------------
+
+// Activation operands of all matrix instructions of one k step (shared by the wave's tiles).
+template <int BITS>
+struct MfmaActivations {
+  u32x4 x[kBlocksPerUnit][BITS == 4 ? 4 : 2];
+};
+
+// Weights, scales and zeros of one unit.
+template <int BITS, int GROUPS_PER_RUN>
+struct MfmaWeights {
+  u32x4 w[kBlocksPerUnit];
+  uint32_t s[GROUPS_PER_RUN];
+  uint32_t z[GROUPS_PER_RUN];
+};
+
+template <int BITS>
+__device__ __forceinline__ void load_activations_mfma(MfmaActivations<BITS>& f, const Problem& p,
+                                                      __amdgpu_buffer_rsrc_t x_rsrc, int kstep, int lane) {
+  using G = Geometry<BITS>;
+  constexpr int kFrags = BITS == 4 ? 4 : 2;  // matrix instructions per block
+  const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
+  const int m = lane % kTileRows;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) {
+    const int k_block = k_run + i * G::kChunkK;
+    // Batch rows past m_batch and reduction positions past k fall outside the descriptor and
+    // read as zero (k is a multiple of the chunk, so a block is wholly inside or outside).
+    const uint32_t off = k_block < p.k ? (uint32_t)(m * p.k + k_block) * 2u : 0xfffffff0u;
+#pragma unroll
+    for (int j = 0; j < kFrags; ++j) f.x[i][j] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, j * 16, kCacheDefault);
+  }
+}
+
+template <int BITS, int QOP, int GROUPS_PER_RUN>
+__device__ __forceinline__ void load_weights_mfma(MfmaWeights<BITS, GROUPS_PER_RUN>& f, const Problem& p,
+                                                  __amdgpu_buffer_rsrc_t w_rsrc, int byte_offset, int kstep, int lane,
+                                                  int row) {
+  using G = Geometry<BITS>;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i)
+    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * kChunkBytes, byte_offset + i * kBlockBytes, kCacheStream);
+  if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) {
+    const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
+      const int grp = group_of(p, k_run + gi * (G::kRunK / GROUPS_PER_RUN));
+      const int idx = grp * p.n_out + row;
+      f.s[gi] = load_half_bits(p.scale + idx);
+      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS) f.z[gi] = load_half_bits(p.zero_add + idx);
+    }
+  }
+}
+
+template <int BITS, int QOP, int GROUPS_PER_RUN>
+__device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
+                                                  const MfmaActivations<BITS>& xa, const ConvertRegs& c,
+                                                  half2_t col_scale2) {
+  constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) {
+    const int gi = i * GROUPS_PER_RUN / kBlocksPerUnit;
+    half2_t s2 = col_scale2, z2 = half2_t{};
+    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) s2 = splat_low(f.s[gi]);
+    if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
+    if constexpr (BITS == 4) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        half2_t q[4];
+        convert_int4_word(f.w[i][j], c, q);
+        u32x4 a;
+#pragma unroll
+        for (int h = 0; h < 4; ++h) a[h] = as_u32(dequant_pair<kHasZero>(q[h], s2, z2));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, xa.x[i][j]),
+                                                     acc, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        half2_t q0[2], q1[2];
+        convert_int8_word(f.w[i][2 * j], c, q0);
+        convert_int8_word(f.w[i][2 * j + 1], c, q1);
+        u32x4 a;
+        a[0] = as_u32(dequant_pair<kHasZero>(q0[0], s2, z2));
+        a[1] = as_u32(dequant_pair<kHasZero>(q0[1], s2, z2));
+        a[2] = as_u32(dequant_pair<kHasZero>(q1[0], s2, z2));
+        a[3] = as_u32(dequant_pair<kHasZero>(q1[1], s2, z2));
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, xa.x[i][j]),
+                                                     acc, 0, 0, 0);
+      }
+    }
+  }
+}
+
+// blockDim = (64 * split_k, tiles_per_wg); each wave works on T consecutive tiles so that the
+// activation operands of a k step are fetched once and used T times.  Dynamic LDS:
+// tiles_per_wg * split_k * T * 256 floats (none when split_k == 1).  m_batch travels in
+// tail.reserved.
+template <int BITS, int QOP, int GROUPS_PER_RUN, int T>
+__global__ void __launch_bounds__(kWave * kMaxWavesPerMfmaWorkgroup)
+gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
+                 uint32_t packed_steps, int workgroups, int wgs_per_xcd, uint32_t packed_group, GemvTail tail) {
+  extern __shared__ float partials[];
+  Problem p;
+  p.weights = weights;
+  p.x = x;
+  p.scale = scale;
+  p.zero_add = zero_add;
+  p.n_out = n_out;
+  p.k = k;
+  p.ksteps = (int)(packed_steps & 0xffffu);
+  p.steps_per_wave = (int)(packed_steps >> 16);
+  p.workgroups = workgroups;
+  p.wgs_per_xcd = wgs_per_xcd;
+  p.group_size = (int)(packed_group & 0xffffffu);
+  p.tiles_per_wg = (int)(packed_group >> 24);
+  asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
+               "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
+               "s"(tail.reserved), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
+               "s"(tail.stride_bias), "s"(tail.stride_y));
+  const long long batch = blockIdx.z;
+  p.weights += batch * tail.stride_weights;
+  p.x += batch * tail.stride_x;
+  p.scale += batch * tail.stride_scale;
+  p.zero_add += batch * tail.stride_scale;
+  const bool has_bias = tail.bias != nullptr;
+  tail.bias += batch * tail.stride_bias;
+  tail.y += batch * tail.stride_y;
+  const int m_batch = tail.reserved;
+
+  const int wg = logical_workgroup(p);
+  if (wg >= p.workgroups) return;
+
+  const int lane = threadIdx.x % kWave;
+  const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);
+  const int tile0 = (wg * p.tiles_per_wg + ty) * T;
+  const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
+  int row[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const int r = (tile0 + t) * kTileRows + lane % kTileRows;
+    row[t] = r < p.n_out ? r : p.n_out - 1;
+  }
+
+  f32x4 acc[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  const int ks_begin = kw * p.steps_per_wave;
+  const int ks_end = min(ks_begin + p.steps_per_wave, p.ksteps);
+  if (tile0 < tiles && ks_begin < ks_end) {
+    const int units = ks_end - ks_begin;
+    const int my_tiles = min(T, tiles - tile0);
+    const int tile_stride = p.ksteps * kUnitBytes;  // bytes from a unit to the same k step of the next tile
+    // One descriptor spans the wave's tiles; tiles past the matrix read as zero.
+    const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
+        p.weights + ((size_t)tile0 * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
+        (uint32_t)(my_tiles - 1) * (uint32_t)tile_stride + (uint32_t)units * (uint32_t)kUnitBytes);
+    const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(p.x, (uint32_t)m_batch * (uint32_t)p.k * 2u);
+    half2_t col_scale[T];
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      col_scale[t] = half2_t{};
+      if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale[t] = splat(p.scale[row[t]]);
+    }
+    const ConvertRegs c = make_convert_regs();
+    for (int u = 0; u < units; ++u) {
+      MfmaActivations<BITS> xa;
+      MfmaWeights<BITS, GROUPS_PER_RUN> wt[T];
+#pragma unroll
+      for (int t = 0; t < T; ++t)
+        load_weights_mfma<BITS, QOP, GROUPS_PER_RUN>(wt[t], p, w_rsrc, t * tile_stride + u * kUnitBytes, ks_begin + u, lane,
+                                                     row[t]);
+      load_activations_mfma<BITS>(xa, p, x_rsrc, ks_begin + u, lane);
+#pragma unroll
+      for (int t = 0; t < T; ++t) compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc[t], wt[t], xa, c, col_scale[t]);
+    }
+  }
+
+  // Lane l holds D[rows 4*(l/16) .. +3 of the tile][batch row l % 16] for each of its tiles.
+  const int split_k = tail.split_k;
+  if (split_k > 1) {
+    f32x4* park = reinterpret_cast<f32x4*>(partials) + ((ty * split_k + kw) * T) * kWave + lane;
+#pragma unroll
+    for (int t = 0; t < T; ++t) park[t * kWave] = acc[t];
+    __syncthreads();
+    if (tile0 >= tiles) return;
+    // wave kw finishes tiles t = kw, kw + split_k, ...
+    for (int t = kw; t < T; t += split_k) {
+      const f32x4* part = reinterpret_cast<const f32x4*>(partials) + (ty * split_k * T + t) * kWave + lane;
+      f32x4 sum = part[0];
+      for (int w = 1; w < split_k; ++w) sum += part[w * T * kWave];
+      const int m = lane % kTileRows;
+      const int n0 = (tile0 + t) * kTileRows + 4 * (lane / kTileRows);
+      if (m < m_batch) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int n = n0 + v;
+          if (n < p.n_out) {
+            float r = sum[v];
+            if (has_bias) r += (float)tail.bias[n];
+            tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
+          }
+        }
+      }
+    }
+    return;
+  }
+  if (tile0 >= tiles) return;
+  const int m = lane % kTileRows;
+  if (m < m_batch) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const int n0 = (tile0 + t) * kTileRows + 4 * (lane / kTileRows);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int n = n0 + v;
+        if (n < p.n_out) {
+          float r = acc[t][v];
+          if (has_bias) r += (float)tail.bias[n];
+          tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
+        }
+      }
+    }
+  }
+}
+
 struct DequantParams {
   const uint8_t* weights;
   const half_t* scale;
@@ -360,37 +601,54 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, 
 
 std::atomic<int> g_override_split_k{0};
 std::atomic<int> g_override_tiles_per_wg{0};
+std::atomic<int> g_override_tiles_per_wave{0};
+std::atomic<int> g_matrix_core_min_batch{5};  // m_batch from which the matrix-core kernel is used
+
+inline bool use_matrix_cores(int m_batch) { return m_batch >= g_matrix_core_min_batch.load(); }
 
 struct LaunchPlan {
   int split_k, tiles_per_wg, steps_per_wave, workgroups, wgs_per_xcd, threads;
+  int tiles_per_wave;  // 1 on the VALU path; 1, 2 or 4 on the matrix-core path
 };
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-LaunchPlan plan_launch(int n_out, int k, int bits) {
+LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
-  // Measured on MI355X: one tile per workgroup and as many k-split waves as the tile has
+  const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
+  const int ov_t = g_override_tiles_per_wave.load();
+  // Matrix-core path: a wave that works on T tiles fetches the activation operands of a k step
+  // once for all of them.  Measured on 8192 x 8192 (512 tiles): T = 2 is 1.5-1.8x faster than
+  // T = 1 at 8-16 activation rows; T = 4 leaves too few waves to cover the load latency.
+  int tiles_per_wave = 1;
+  if (use_matrix_cores(m_batch)) {
+    tiles_per_wave = tiles >= 256 ? 2 : 1;
+    if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
+  }
+  const int groups = ceil_div(tiles, tiles_per_wave);
+  // Measured on MI355X: one tile (group) per workgroup and as many k-split waves as there are
   // units (at most 16) is best or within a few percent of best for every shape tried, until
   // the launch exceeds ~16k waves; beyond that halve the split so each wave keeps >= 2 units.
   constexpr int kWaveBudget = 16384;
-  int split_k = ksteps < kMaxWavesPerWorkgroup ? ksteps : kMaxWavesPerWorkgroup;
-  while (split_k > 1 && (long long)tiles * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
+  const int max_waves = use_matrix_cores(m_batch) ? kMaxWavesPerMfmaWorkgroup : kMaxWavesPerWorkgroup;
+  int split_k = ksteps < max_waves ? ksteps : max_waves;
+  while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
   int tiles_per_wg = 1;
-  const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
   if (ov_sk > 0) split_k = ov_sk;
   if (ov_tw > 0) tiles_per_wg = ov_tw;
-  split_k = split_k > kMaxWavesPerWorkgroup ? kMaxWavesPerWorkgroup : split_k;
+  split_k = split_k > max_waves ? max_waves : split_k;
   split_k = split_k > ksteps ? ksteps : split_k;
   const int steps = ceil_div(ksteps, split_k);
   split_k = ceil_div(ksteps, steps);
-  if (tiles_per_wg * split_k > kMaxWavesPerWorkgroup) tiles_per_wg = kMaxWavesPerWorkgroup / split_k;
+  if (tiles_per_wg * split_k > max_waves) tiles_per_wg = max_waves / split_k;
   LaunchPlan lp;
   lp.split_k = split_k;
   lp.tiles_per_wg = tiles_per_wg;
   lp.steps_per_wave = steps;
-  lp.workgroups = ceil_div(tiles, tiles_per_wg);
+  lp.workgroups = ceil_div(groups, tiles_per_wg);
   lp.wgs_per_xcd = ceil_div(lp.workgroups, kNumXcd);
   lp.threads = kWave * split_k * tiles_per_wg;
+  lp.tiles_per_wave = tiles_per_wave;
   return lp;
 }
 
@@ -495,6 +753,50 @@ hipError_t launch_gemv(const GemvLaunch& g, int bits, int qop, int mb, int gpr) 
   }
 }
 
+template <int BITS, int QOP, int GPR, int T>
+hipError_t launch_mfma_kernel_t(const GemvLaunch& g) {
+  return launch(gemv_mfma_kernel<BITS, QOP, GPR, T>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
+                g.zero_add, g.n_out, g.k, pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups,
+                g.plan.wgs_per_xcd, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+}
+
+template <int BITS, int QOP, int GPR>
+hipError_t launch_mfma_kernel(const GemvLaunch& g) {
+  switch (g.plan.tiles_per_wave) {
+    case 1: return launch_mfma_kernel_t<BITS, QOP, GPR, 1>(g);
+    case 2: return launch_mfma_kernel_t<BITS, QOP, GPR, 2>(g);
+    default: return launch_mfma_kernel_t<BITS, QOP, GPR, 4>(g);
+  }
+}
+
+template <int BITS, int QOP>
+hipError_t launch_mfma_gpr(const GemvLaunch& g, int gpr) {
+  if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+    return launch_mfma_kernel<BITS, QOP, 1>(g);
+  } else {
+    switch (gpr) {
+      case 1: return launch_mfma_kernel<BITS, QOP, 1>(g);
+      case 2: return launch_mfma_kernel<BITS, QOP, 2>(g);
+      default: return launch_mfma_kernel<BITS, QOP, 4>(g);
+    }
+  }
+}
+
+hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr) {
+  if (bits == 4) {
+    switch (qop) {
+      case 1: return launch_mfma_gpr<4, 1>(g, gpr);
+      case 2: return launch_mfma_gpr<4, 2>(g, gpr);
+      default: return launch_mfma_gpr<4, 3>(g, gpr);
+    }
+  }
+  switch (qop) {
+    case 1: return launch_mfma_gpr<8, 1>(g, gpr);
+    case 2: return launch_mfma_gpr<8, 2>(g, gpr);
+    default: return launch_mfma_gpr<8, 3>(g, gpr);
+  }
+}
+
 template <int BITS>
 hipError_t launch_dequant(const DequantParams& p, int qop, half_t* out, hipStream_t stream) {
   const long long units = (long long)p.tiles * p.ksteps;
@@ -531,7 +833,7 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.n_out = n_out;
   g.k = k;
   g.group_size = group_size;
-  g.plan = plan_launch(n_out, k, weight_bits);
+  g.plan = plan_launch(n_out, k, weight_bits, m_batch);
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.stride_weights = stride_weights;
@@ -544,7 +846,15 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.stream = static_cast<hipStream_t>(stream);
   const int gpr = groups_per_run(group_size, weight_bits);
 
-  // Activation rows are processed kMaxValuBatch at a time.
+  if (use_matrix_cores(m_batch)) {
+    g.x = reinterpret_cast<const half_t*>(x);
+    g.tail.y = reinterpret_cast<half_t*>(y);
+    g.tail.reserved = m_batch;
+    g.lds = g.plan.split_k == 1 ? 0
+                                : (size_t)g.plan.tiles_per_wg * g.plan.split_k * g.plan.tiles_per_wave * kWave * 4 * sizeof(float);
+    return launch_mfma(g, weight_bits, quant_op, gpr) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+  }
+  // VALU path: activation rows are processed kMaxValuBatch at a time.
   for (int m0 = 0; m0 < m_batch; m0 += kMaxValuBatch) {
     const int mb = m_batch - m0 < kMaxValuBatch ? m_batch - m0 : kMaxValuBatch;
     g.x = reinterpret_cast<const half_t*>(x) + (size_t)m0 * (size_t)k;
@@ -583,25 +893,34 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
   return e == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
 }
 
-int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup) {
-  if (split_k_waves < 0 || tiles_per_workgroup < 0) return MGEMV_ERR_SIZE;
+int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave) {
+  if (split_k_waves < 0 || tiles_per_workgroup < 0 || tiles_per_wave < 0) return MGEMV_ERR_SIZE;
+  if (tiles_per_wave != 0 && tiles_per_wave != 1 && tiles_per_wave != 2 && tiles_per_wave != 4) return MGEMV_ERR_SIZE;
   mgemv::g_override_split_k.store(split_k_waves);
   mgemv::g_override_tiles_per_wg.store(tiles_per_workgroup);
+  mgemv::g_override_tiles_per_wave.store(tiles_per_wave);
   return MGEMV_OK;
 }
 
-int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[6]) {
+int mgemv_set_matrix_core_threshold(int min_m_batch) {
+  if (min_m_batch < 0 || min_m_batch > MGEMV_MAX_M_BATCH + 1) return MGEMV_ERR_BATCH;
+  mgemv::g_matrix_core_min_batch.store(min_m_batch == 0 ? 5 : min_m_batch);
+  return MGEMV_OK;
+}
+
+int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[7]) {
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
   if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
-  const mgemv::LaunchPlan lp = mgemv::plan_launch(n_out, k, weight_bits);
+  const mgemv::LaunchPlan lp = mgemv::plan_launch(n_out, k, weight_bits, m_batch);
   out[0] = lp.wgs_per_xcd * mgemv::kNumXcd;
   out[1] = lp.threads;
   out[2] = lp.split_k;
   out[3] = lp.tiles_per_wg;
   out[4] = lp.steps_per_wave;
-  out[5] = 0;
+  out[5] = mgemv::use_matrix_cores(m_batch) ? 1 : 0;
+  out[6] = lp.tiles_per_wave;
   return MGEMV_OK;
 }
 
