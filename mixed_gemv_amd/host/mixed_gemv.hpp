@@ -1,0 +1,187 @@
+// C++ host-side mirror of the reference's call sites on top of the C-ABI (include/mixed_gemv.h).
+//
+// A caller of JJXiangJiaoJun/mixed_gemv uses three things: the host utilities of
+// utils/preprocess.h (SubBytePacker, ZeroPointPreprocessor, MixedGemvWeightPreprocessor), the
+// device adaptor of gemv/device/gemv_adaptor.h (Arguments / initialize / run), and the
+// device_gemv wrapper of mixed_gemv_test.cu:124-165.  The classes below keep those names,
+// argument orders and meanings, so a port is a change of namespace and of the half type
+// (fp16 crosses this interface as uint16_t bit patterns; `half_t` here is that alias).
+//
+// Differences a caller sees, all deliberate:
+//   * the quantisation mode and weight width are run-time constructor arguments of
+//     GemvAdaptor (template parameters in the reference, one binary per mode);
+//   * MixedGemvWeightPreprocessor::run writes preprocessed_size() bytes, which can exceed the
+//     input size (rows padded to 16, k to one wave step); the layout is the gfx950 tile
+//     layout, not RowMajorTileInterleave<8,4>;
+//   * where the reference prints a message and calls exit(-1), these throw mixed_gemv::Error
+//     carrying the C-ABI status (define MIXED_GEMV_EXIT_ON_ERROR to get print + exit(-1)).
+#ifndef MIXED_GEMV_AMD_HOST_MIXED_GEMV_HPP_
+#define MIXED_GEMV_AMD_HOST_MIXED_GEMV_HPP_
+
+#include <cstdint>
+#include <cstdlib>
+#include <iostream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "mixed_gemv.h"
+
+namespace mixed_gemv {
+
+using half_t = uint16_t;  // IEEE binary16 bit pattern
+
+// gemv/weight_only_quant_op.h:12-18
+enum class WeightOnlyQuantOp { UNDEFINED = 0, PER_COLUMN_SCALE_ONLY = 1, FINEGRAINED_SCALE_ONLY = 2, FINEGRAINED_SCALE_AND_ZEROS = 3 };
+constexpr bool isFinegrained(WeightOnlyQuantOp op) { return op == WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS || op == WeightOnlyQuantOp::FINEGRAINED_SCALE_ONLY; }
+constexpr bool hasZero(WeightOnlyQuantOp op) { return op == WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS; }
+
+// utils/type_base.h:7-16
+enum class QuantType { W8_A16 = 0, W4_A16 = 1, W4_AFP8 = 2 };
+enum class LayoutType { kRowMajor = 0, kColumnMajor = 1 };
+
+class Error : public std::runtime_error {
+ public:
+  Error(int status, const std::string& where)
+      : std::runtime_error(where + ": " + mgemv_status_string(status)), status_(status) {}
+  int status() const { return status_; }
+
+ private:
+  int status_;
+};
+
+inline void check(int status, const char* where) {
+  if (status == MGEMV_OK) return;
+#ifdef MIXED_GEMV_EXIT_ON_ERROR
+  std::cout << where << ": " << mgemv_status_string(status) << std::endl;
+  std::exit(-1);
+#else
+  throw Error(status, where);
+#endif
+}
+
+// utils/preprocess.h:16-85
+struct SubBytePacker {
+  static void unpack(int8_t* unpacked_output, const int8_t* packed_input, size_t packed_num_elements) {
+    check(mgemv_unpack_int4(unpacked_output, reinterpret_cast<const uint8_t*>(packed_input), packed_num_elements), "SubBytePacker::unpack");
+  }
+  static void pack(int8_t* packed_output, const int8_t* unpacked_input, size_t unpacked_num_elements) {
+    check(mgemv_pack_int4(reinterpret_cast<uint8_t*>(packed_output), unpacked_input, unpacked_num_elements), "SubBytePacker::pack");
+  }
+};
+
+// utils/preprocess.h:88-102
+struct ZeroPointPreprocessor {
+  static void neg_zero_point_multiplies_scale(half_t* neg_zeros_x_scales, const half_t* scales, const int8_t* zeros, int n) {
+    check(mgemv_fold_zero_points(neg_zeros_x_scales, scales, zeros, static_cast<size_t>(n)), "ZeroPointPreprocessor");
+  }
+};
+
+// utils/preprocess.h:480-524
+struct MixedGemvWeightPreprocessor {
+  static size_t preprocessed_size(const std::vector<size_t>& shape, QuantType quant_type) {
+    return mgemv_preprocessed_size(shape.data(), static_cast<int>(shape.size()), static_cast<int>(quant_type));
+  }
+  // shape = {K, M} or {experts, K, M}; preprocessed_quantized_weight must hold preprocessed_size() bytes.
+  static void run(int8_t* preprocessed_quantized_weight, const int8_t* quantized_weight, const std::vector<size_t>& shape,
+                  LayoutType weight_layout, QuantType quant_type, bool /*force_interleave: ignored, as in the reference*/) {
+    check(mgemv_preprocess_weights(reinterpret_cast<uint8_t*>(preprocessed_quantized_weight),
+                                   reinterpret_cast<const uint8_t*>(quantized_weight), shape.data(),
+                                   static_cast<int>(shape.size()), static_cast<int>(weight_layout), static_cast<int>(quant_type)),
+          "MixedGemvWeightPreprocessor::run");
+  }
+};
+
+struct GemmCoord {
+  int m_, n_, k_;
+  int m() const { return m_; }
+  int n() const { return n_; }
+  int k() const { return k_; }
+};
+
+template <typename T>
+struct TensorRef {
+  T* ptr;
+  int ld;
+  T* data() const { return ptr; }
+  int stride() const { return ld; }
+};
+
+// gemv/device/gemv_adaptor.h:114-261.  Reference letters: M = output features, N = activation
+// rows, K = reduction.  The leading dimensions are accepted for source compatibility; the
+// kernels use dense operands (scale/zero/C/D with ld = M, activations with row stride K).
+class GemvAdaptor {
+ public:
+  struct Arguments {
+    GemmCoord problem_size;
+    TensorRef<const void> ref_A;             // PREPROCESSED weights
+    TensorRef<const half_t> ref_B;           // activations
+    TensorRef<const half_t> ref_scale;
+    TensorRef<const half_t> ref_zero_point;  // folded -z*s
+    TensorRef<const half_t> ref_C;           // optional bias, nullptr = none
+    TensorRef<half_t> ref_D;
+    int group_size = 64;
+    int batch_count = 1;
+    long long batch_stride_A = 0;            // BYTES of the preprocessed buffer
+    long long batch_stride_B = 0, batch_stride_scale = 0, batch_stride_C = 0, batch_stride_D = 0;  // elements
+  };
+
+  GemvAdaptor(WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4)
+      : quant_op_(quant_op), weight_bits_(weight_bits) {}
+
+  void initialize(const Arguments& args, void* /*stream*/ = nullptr) {
+    // gemv_adaptor.h:199-203
+    if (quant_op_ != WeightOnlyQuantOp::PER_COLUMN_SCALE_ONLY && args.group_size < 64) check(MGEMV_ERR_GROUP_SIZE, "GemvAdaptor::initialize");
+    args_ = args;
+    initialized_ = true;
+  }
+
+  void run(void* stream = nullptr) {
+    if (!initialized_) throw std::logic_error("GemvAdaptor::run before initialize");
+    const Arguments& a = args_;
+    const half_t* zero = hasZero(quant_op_) ? a.ref_zero_point.ptr : nullptr;  // mixed_gemv_test.cu:145-147
+    check(mgemv_gemv_batched(a.ref_A.ptr, a.ref_B.ptr, a.ref_scale.ptr, zero, a.ref_C.ptr, a.ref_D.ptr, a.batch_count,
+                             a.problem_size.m(), a.problem_size.n(), a.problem_size.k(), a.group_size,
+                             static_cast<int>(quant_op_), weight_bits_, a.batch_stride_A, a.batch_stride_B,
+                             a.batch_stride_scale, a.batch_stride_C, a.batch_stride_D, stream),
+          "GemvAdaptor::run");
+  }
+
+  void operator()(const Arguments& args, void* stream = nullptr) {
+    initialize(args, stream);
+    run(stream);
+  }
+
+ private:
+  WeightOnlyQuantOp quant_op_;
+  int weight_bits_;
+  Arguments args_{};
+  bool initialized_ = false;
+};
+
+// mixed_gemv_test.cu:124-165.  Same argument order; the quant mode, a compile-time constant in
+// the reference, and the stream are trailing arguments.
+inline void device_gemv(const void* ptr_A, const half_t* ptr_B, const half_t* ptr_scale, const half_t* ptr_zero_point,
+                        const half_t* ptr_C, half_t* ptr_D, int B, int M, int N, int K, int group_size,
+                        WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4,
+                        void* stream = nullptr) {
+  if (quant_op == WeightOnlyQuantOp::PER_COLUMN_SCALE_ONLY) group_size = K;            // :142-143
+  if (quant_op != WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS) ptr_zero_point = nullptr;  // :145-147
+  GemvAdaptor::Arguments args;
+  args.problem_size = GemmCoord{M, N, K};
+  args.ref_A = {ptr_A, K * 4};
+  args.ref_B = {ptr_B, 0};
+  args.ref_scale = {ptr_scale, M};
+  args.ref_zero_point = {ptr_zero_point, M};
+  args.ref_C = {ptr_C, M};
+  args.ref_D = {ptr_D, M};
+  args.group_size = group_size;
+  args.batch_count = B;
+  GemvAdaptor op(quant_op, weight_bits);
+  op.initialize(args);
+  op.run(stream);
+}
+
+}  // namespace mixed_gemv
+
+#endif  // MIXED_GEMV_AMD_HOST_MIXED_GEMV_HPP_
