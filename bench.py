@@ -75,18 +75,36 @@ class Workload:
         qt = mg.QuantType.W4_A16 if self.bits == 4 else mg.QuantType.W8_A16
         self.raw0 = None
         self.w, self.s, self.z = [], [], []
+        # All rotating sets live in ONE device allocation (256-byte aligned slices): large
+        # contiguous mappings keep address-translation misses on cold buffers low.
+        w_bytes = mg.preprocessed_size((self.k, self.n_out), qt)
+        s_bytes = groups * self.n_out * 2
+        align = lambda v: (v + 255) // 256 * 256  # noqa: E731
+        set_bytes = align(w_bytes) + 2 * align(s_bytes)
+        self.arena = torch.empty(set_bytes * self.sets, dtype=torch.uint8, device=device)
+
+        def carve(offset, nbytes, dtype, shape):
+            return self.arena[offset:offset + nbytes].view(dtype).view(shape)
+
         for i in range(self.sets):
+            base = i * set_bytes
             # uniform random bytes == uniform int4 pairs in [-8, 7] (or int8 in [-128, 127])
             raw = torch.randint(0, 256, (self.n_out * self.k * self.bits // 8,), dtype=torch.uint8, generator=gen)
             if i == 0:
                 self.raw0 = raw.numpy().copy()
             pre = mg.MixedGemvWeightPreprocessor.run(raw.numpy(), (self.k, self.n_out), mg.LayoutType.kColumnMajor, qt)
-            self.w.append(torch.from_numpy(pre).to(device))
+            w = carve(base, w_bytes, torch.uint8, (w_bytes,))
+            w.copy_(torch.from_numpy(pre))
+            self.w.append(w)
             sc = (torch.rand((groups, self.n_out), generator=gen) * (srange[1] - srange[0]) + srange[0]).half()
-            self.s.append(sc.to(device))
+            sdev = carve(base + align(w_bytes), s_bytes, torch.half, (groups, self.n_out))
+            sdev.copy_(sc)
+            self.s.append(sdev)
             if self.quant_op == 3:
                 zz = (torch.rand((groups, self.n_out), generator=gen) * 0.1 - 0.05).half()
-                self.z.append(zz.to(device))
+                zdev = carve(base + align(w_bytes) + align(s_bytes), s_bytes, torch.half, (groups, self.n_out))
+                zdev.copy_(zz)
+                self.z.append(zdev)
             else:
                 self.z.append(None)
         if xdist == "uniform":

@@ -35,6 +35,8 @@ struct GemvTail {
   const half_t* bias;
   half_t* y;
   int split_k;         // waves of a workgroup that share one tile (blockDim.x / 64)
+  int m_batch;         // activation rows (matrix-core kernel)
+  int num_groups;      // k / group_size (1 in per-column mode): extent of the scale / zero tables
   int reserved;
   long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
 };
@@ -93,33 +95,92 @@ __device__ __forceinline__ half2_t splat_low(uint32_t bits) {
   return half2_t{h, h};
 }
 
+// Where a lane reads for the current unit.  Everything that varies along k sits in the VGPR
+// offset of the buffer loads (the part of the address that the hardware bounds-checks), so
+// reads past k or past the last group return zero instead of touching foreign memory.
+//
+// GROUPS_PER_RUN 1 or 2 ("regular"): the group size divides the k step, so a lane's scale /
+// zero offset just advances by a constant per unit.  GROUPS_PER_RUN 4 ("generic", any group
+// size that is a multiple of 32): one lookup per block with an integer division.
+template <int BITS, int GROUPS_PER_RUN>
+struct WaveCursor {
+  int w_voffset;                   // byte offset of this lane's chunk of block 0 inside the wave's weight range
+  int x_voffset;                   // byte offset of this lane's activations
+  int sz_voffset[GROUPS_PER_RUN];  // regular: byte offset of this lane's scale / zero
+  int k_run;                       // generic: first reduction index of the lane's run
+  int sz_stride;                   // regular: bytes per k step in the scale / zero tables
+};
+
+template <int BITS, int GROUPS_PER_RUN>
+__device__ __forceinline__ WaveCursor<BITS, GROUPS_PER_RUN> make_cursor(const Problem& p, int ks_begin, int lane, int row) {
+  using G = Geometry<BITS>;
+  WaveCursor<BITS, GROUPS_PER_RUN> c;
+  c.w_voffset = lane * kChunkBytes;
+  c.x_voffset = ks_begin * (G::kStepK * 2) + lane * (BITS == 4 ? 16 : 8);
+  c.k_run = ks_begin * G::kStepK + (lane / kTileRows) * G::kRunK;
+  if constexpr (GROUPS_PER_RUN != 4) {
+    // Regular modes: the group size divides the k step, hence is a power of two; no divisions.
+    const int shift = __builtin_ctz((unsigned)p.group_size);
+    const int groups_per_step = G::kStepK >> shift;
+    c.sz_stride = groups_per_step * p.n_out * 2;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
+      const int k_local = (lane / kTileRows) * G::kRunK + gi * (G::kRunK / GROUPS_PER_RUN);
+      c.sz_voffset[gi] = ((ks_begin * groups_per_step + (k_local >> shift)) * p.n_out + row) * 2;
+    }
+  } else {
+    c.sz_stride = 0;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) c.sz_voffset[gi] = 0;
+  }
+  return c;
+}
+
+template <int BITS, int GROUPS_PER_RUN>
+__device__ __forceinline__ void advance(WaveCursor<BITS, GROUPS_PER_RUN>& c) {
+  using G = Geometry<BITS>;
+  c.w_voffset += kUnitBytes;
+  c.x_voffset += G::kStepK * 2;
+  c.k_run += G::kStepK;
+#pragma unroll
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) c.sz_voffset[gi] += c.sz_stride;
+}
+
+struct ScaleTables {
+  __amdgpu_buffer_rsrc_t scale, zero;
+};
+
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f, const Problem& p,
                                           __amdgpu_buffer_rsrc_t w_rsrc, const __amdgpu_buffer_rsrc_t (&x_rsrc)[MB],
-                                          int unit_in_wave, int kstep, int lane, int row) {
+                                          const ScaleTables& tables, const WaveCursor<BITS, GROUPS_PER_RUN>& c, int lane,
+                                          int row) {
   using G = Geometry<BITS>;
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i)
-    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * kChunkBytes,
-                                                   unit_in_wave * kUnitBytes + i * kBlockBytes, kCacheStream);
+    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c.w_voffset + i * kBlockBytes, 0, kCacheStream);
 #pragma unroll
   for (int m = 0; m < MB; ++m) {
     if constexpr (BITS == 4) {
-      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc[m], lane * 16, kstep * (G::kStepK * 2), kCacheDefault);
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc[m], c.x_voffset, 0, kCacheDefault);
       f.x[m][0] = v[0]; f.x[m][1] = v[1]; f.x[m][2] = v[2]; f.x[m][3] = v[3];
     } else {
-      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc[m], lane * 8, kstep * (G::kStepK * 2), kCacheDefault);
+      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc[m], c.x_voffset, 0, kCacheDefault);
       f.x[m][0] = v[0]; f.x[m][1] = v[1];
     }
   }
   if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) {
-    const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
 #pragma unroll
     for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
-      const int grp = group_of(p, k_run + gi * (G::kRunK / GROUPS_PER_RUN));
-      const int idx = grp * p.n_out + row;
-      f.s[gi] = load_half_bits(p.scale + idx);
-      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS) f.z[gi] = load_half_bits(p.zero_add + idx);
+      int voffset;
+      if constexpr (GROUPS_PER_RUN == 4) {
+        voffset = (group_of(p, c.k_run + gi * G::kChunkK) * p.n_out + row) * 2;
+      } else {
+        voffset = c.sz_voffset[gi];
+      }
+      f.s[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.scale, voffset, 0, kCacheDefault);
+      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS)
+        f.z[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.zero, voffset, 0, kCacheDefault);
     }
   }
 }
@@ -207,8 +268,8 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   // load-wait pairs in front of the first weight load of these microsecond-scale kernels.
   asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
                "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
-               "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale), "s"(tail.stride_bias),
-               "s"(tail.stride_y));
+               "s"(tail.num_groups), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
+               "s"(tail.stride_bias), "s"(tail.stride_y));
   // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223); branch-free.
   const long long batch = blockIdx.z;
   p.weights += batch * tail.stride_weights;
@@ -245,21 +306,39 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
 #pragma unroll
     for (int m = 0; m < MB; ++m) x_rsrc[m] = make_rsrc(p.x + (size_t)m * (size_t)p.k, (uint32_t)p.k * 2u);
 
+    ScaleTables tables;
+    const uint32_t table_bytes = (uint32_t)tail.num_groups * (uint32_t)p.n_out * 2u;
+    tables.scale = make_rsrc(p.scale, table_bytes);
+    tables.zero = make_rsrc(p.zero_add, QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? table_bytes : 0u);
+    WaveCursor<BITS, GROUPS_PER_RUN> cur = make_cursor<BITS, GROUPS_PER_RUN>(p, ks_begin, lane, row);
+
     // Two fragments in flight: the loads of unit u+1 are issued before unit u is computed, so
     // a wave that is waiting for its turn on the VALU still has memory requests outstanding.
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
-    load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, 0, ks_begin, lane, row);
+    load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur, lane, row);
     half2_t col_scale = half2_t{};
     if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = splat(p.scale[row]);
     const ConvertRegs c = make_convert_regs();
-    int u = 0;
-    while (true) {
-      if (u + 1 < units) load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, u + 1, ks_begin + u + 1, lane, row);
+    if (units == 1) {
       compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale);
-      if (++u >= units) break;
-      if (u + 1 < units) load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, u + 1, ks_begin + u + 1, lane, row);
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, col_scale);
-      if (++u >= units) break;
+    } else {
+      // The prefetches are unconditional: past the wave's last unit every offset is out of the
+      // descriptors' range, the loads return zero without touching memory, and the compiler
+      // can count outstanding loads exactly instead of draining them all before each use.
+      int u = 0;
+      do {
+        advance(cur);
+        load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur, lane, row);
+        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
+        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale);
+        advance(cur);
+        __builtin_amdgcn_sched_barrier(0);
+        load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur, lane, row);
+        __builtin_amdgcn_sched_barrier(0);
+        if (u + 1 < units) compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, col_scale);
+        __builtin_amdgcn_sched_barrier(0);
+        u += 2;
+      } while (u < units);
     }
 #pragma unroll
     for (int m = 0; m < MB; ++m) settle_dot_chain(acc[m]);
@@ -428,7 +507,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   p.tiles_per_wg = (int)(packed_group >> 24);
   asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
                "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
-               "s"(tail.reserved), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
+               "s"(tail.m_batch), "s"(tail.num_groups), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
                "s"(tail.stride_bias), "s"(tail.stride_y));
   const long long batch = blockIdx.z;
   p.weights += batch * tail.stride_weights;
@@ -438,7 +517,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   const bool has_bias = tail.bias != nullptr;
   tail.bias += batch * tail.stride_bias;
   tail.y += batch * tail.stride_y;
-  const int m_batch = tail.reserved;
+  const int m_batch = tail.m_batch;
 
   const int wg = logical_workgroup(p);
   if (wg >= p.workgroups) return;
@@ -464,7 +543,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
     const int units = ks_end - ks_begin;
     const int my_tiles = min(T, tiles - tile0);
     const int tile_stride = p.ksteps * kUnitBytes;  // bytes from a unit to the same k step of the next tile
-    // One descriptor spans the wave's tiles; tiles past the matrix read as zero.
+    // One descriptor spans the wave's tiles.
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
         p.weights + ((size_t)tile0 * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
         (uint32_t)(my_tiles - 1) * (uint32_t)tile_stride + (uint32_t)units * (uint32_t)kUnitBytes);
@@ -481,8 +560,8 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
       MfmaWeights<BITS, GROUPS_PER_RUN> wt[T];
 #pragma unroll
       for (int t = 0; t < T; ++t)
-        load_weights_mfma<BITS, QOP, GROUPS_PER_RUN>(wt[t], p, w_rsrc, t * tile_stride + u * kUnitBytes, ks_begin + u, lane,
-                                                     row[t]);
+        load_weights_mfma<BITS, QOP, GROUPS_PER_RUN>(wt[t], p, w_rsrc, min(t, my_tiles - 1) * tile_stride + u * kUnitBytes,
+                                                     ks_begin + u, lane, row[t]);  // tiles past the matrix re-read the last one; never stored
       load_activations_mfma<BITS>(xa, p, x_rsrc, ks_begin + u, lane);
 #pragma unroll
       for (int t = 0; t < T; ++t) compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc[t], wt[t], xa, c, col_scale[t]);
@@ -626,13 +705,27 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
     if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
   }
   const int groups = ceil_div(tiles, tiles_per_wave);
-  // Measured on MI355X: one tile (group) per workgroup and as many k-split waves as there are
-  // units (at most 16) is best or within a few percent of best for every shape tried, until
-  // the launch exceeds ~16k waves; beyond that halve the split so each wave keeps >= 2 units.
-  constexpr int kWaveBudget = 16384;
+  // Measured on MI355X with the software-pipelined kernels (one tile group per workgroup is
+  // best throughout):
+  //  * about one workgroup per compute unit or fewer (<= 384 tile groups): few, longer waves --
+  //    4 k-split waves, each pipelining two or more units -- beat more, shorter ones
+  //    (4096x4096: 4.37 us at 4 waves vs 4.57 us at 8);
+  //  * more tile groups than that: split as far as the units allow (at most 16 waves) while the
+  //    launch stays under ~8k waves, and fall back to two units per wave when that still
+  //    leaves >= 4096 waves (8192x8192: 10.6 us at 8 waves vs 11.2 us at 16).
   const int max_waves = use_matrix_cores(m_batch) ? kMaxWavesPerMfmaWorkgroup : kMaxWavesPerWorkgroup;
-  int split_k = ksteps < max_waves ? ksteps : max_waves;
-  while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
+  int split_k;
+  if (groups <= 384) {
+    split_k = ksteps < 4 ? ksteps : 4;
+    if (use_matrix_cores(m_batch)) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
+  } else {
+    constexpr int kWaveBudget = 8192;
+    split_k = ksteps < max_waves ? ksteps : max_waves;
+    while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
+    if (!use_matrix_cores(m_batch) && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
+        (long long)groups * ((split_k + 1) / 2) >= 4096)
+      split_k = (split_k + 1) / 2;
+  }
   int tiles_per_wg = 1;
   if (ov_sk > 0) split_k = ov_sk;
   if (ov_tw > 0) tiles_per_wg = ov_tw;
@@ -679,11 +772,12 @@ int check_problem(const void* weights, const void* scale, const void* zero_add, 
   return MGEMV_OK;
 }
 
+// 1 or 2: the group size divides the k step ("regular" scale addressing, one or two groups per
+// lane run); 4: any other legal group size ("generic", one lookup per block).
 int groups_per_run(int group_size, int bits) {
   const int run = run_k(bits);
-  if (group_size % run == 0) return 1;
-  if (group_size % (run / 2) == 0) return 2;
-  return 4;
+  if (step_k(bits) % group_size != 0) return 4;
+  return group_size % run == 0 ? 1 : 2;
 }
 
 // Launches through hipLaunchKernel so that the status returned is this launch's own, not a
@@ -836,6 +930,7 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.plan = plan_launch(n_out, k, weight_bits, m_batch);
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
+  g.tail.num_groups = k / group_size;
   g.tail.stride_weights = stride_weights;
   g.tail.stride_x = stride_x;
   g.tail.stride_scale = stride_scale;
@@ -849,7 +944,7 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   if (use_matrix_cores(m_batch)) {
     g.x = reinterpret_cast<const half_t*>(x);
     g.tail.y = reinterpret_cast<half_t*>(y);
-    g.tail.reserved = m_batch;
+    g.tail.m_batch = m_batch;
     g.lds = g.plan.split_k == 1 ? 0
                                 : (size_t)g.plan.tiles_per_wg * g.plan.split_k * g.plan.tiles_per_wave * kWave * 4 * sizeof(float);
     return launch_mfma(g, weight_bits, quant_op, gpr) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
