@@ -45,6 +45,21 @@ WORKLOADS = {
 }
 
 
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch,
+# averaged over the launches of `bench.py --workload <name> --launch stream`), scaled by what the same
+# counters read for a plain 512 MiB device copy on the same box: FETCH_SIZE reads 262155.5 for 524288 KiB
+# (factor 2.0), WRITE_SIZE reads 524288 (factor 1.0).  See profiles/.  name -> (fetch KiB raw, write KiB raw)
+MEASURED_TRAFFIC_KIB = {"ns": (4460.5, 8.0), "c5": (61068.5, 56.0)}
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+
+
+def measured_traffic_bytes(name, m_batch):
+    if name not in MEASURED_TRAFFIC_KIB or m_batch != 1:
+        return None
+    fetch, write = MEASURED_TRAFFIC_KIB[name]
+    return int((fetch * FETCH_SCALE + write * WRITE_SCALE) * 1024)
+
+
 def algorithmic_bytes(n_out, k, bits, quant_op, group, m_batch, bias):
     groups = 1 if quant_op == 1 else k // group
     return (n_out * k * bits // 8 + groups * n_out * 2 * (2 if quant_op == 3 else 1) + (n_out * 2 if bias else 0)
@@ -131,44 +146,69 @@ class Workload:
             bias=self.bias.cpu().numpy() if self.bias is not None else None)
 
 
-def time_workload(wl, steps, warmup, use_graph=False):
-    """Returns (wall seconds for `steps` steps, average kernel microseconds by HIP events)."""
+SPIN_UP_SECONDS = 0.06  # the clocks of an idle MI355X take ~20 ms of load to settle (measured: 30.7 -> 25.5 us)
+
+
+def _capture(wl, first, count):
+    """A HIP graph of `count` launches (steps first .. first+count-1): kernel nodes only."""
     import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(first, first + count):
+                wl.launch(i)
+    torch.cuda.current_stream().wait_stream(side)
+    return graph
+
+
+def time_workload(wl, steps, warmup, use_graph=False):
+    """Runs at least `warmup` untimed steps (more if needed to bring an idle device up to its
+    steady clocks), then times EXACTLY `steps` steps.  Returns (wall seconds, average kernel
+    microseconds by a HIP event pair on the launch stream, steps, warm-up steps actually run)."""
+    import torch
+    main = rest = None
+    if use_graph:
+        # whole rotations of the buffer sets, at least 32 kernel nodes per replay so that the cost
+        # of starting a replay is spread thin; a second graph holds the remainder so that the
+        # timed region is exactly `steps` launches
+        nodes = min(steps, wl.sets * max(1, -(-32 // wl.sets)))
+        main = _capture(wl, 0, nodes)
+        if steps % nodes:
+            rest = _capture(wl, 0, steps % nodes)
+    done = 0
     for i in range(warmup):
         wl.launch(i)
+    done += warmup
     torch.cuda.synchronize()
-    graph = None
-    if use_graph:
-        # whole rotations of the buffer sets (at least 32 kernel nodes, so that the cost of starting
-        # a replay is spread thin) captured once, replayed; launches only, no memsets
-        nodes = wl.sets * max(1, -(-32 // wl.sets))
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(graph, stream=side):
-                for i in range(nodes):
-                    wl.launch(i)
-        torch.cuda.current_stream().wait_stream(side)
-        graph.replay()
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < SPIN_UP_SECONDS:
+        if main is not None:
+            main.replay()
+            done += nodes
+        else:
+            for i in range(32):
+                wl.launch(i)
+            done += 32
         torch.cuda.synchronize()
-        replays = max(1, steps // nodes)
-        steps = replays * nodes
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     e0.record()
-    if graph is not None:
-        for _ in range(replays):
-            graph.replay()
+    if main is not None:
+        for _ in range(steps // nodes):
+            main.replay()
+        if rest is not None:
+            rest.replay()
     else:
         for i in range(steps):
             wl.launch(i)
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, e0.elapsed_time(e1) * 1e3 / steps, steps
+    return wall, e0.elapsed_time(e1) * 1e3 / steps, steps, done
 
 
 def check_against_oracle(wl, rows=None):
@@ -211,8 +251,8 @@ def check_against_oracle(wl, rows=None):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=20000)
+    ap.add_argument("--warmup", type=int, default=2000)
     ap.add_argument("--workload", default="ns", choices=sorted(WORKLOADS))
     ap.add_argument("--m-batch", type=int, default=None)
     ap.add_argument("--launch", default="graph", choices=["graph", "stream"],
@@ -235,7 +275,7 @@ def main():
     torch.cuda.set_device(device)
 
     wl = Workload(args.workload, device, m_batch=args.m_batch)
-    wall, ev_us, steps = time_workload(wl, args.steps, args.warmup, use_graph=(args.launch == "graph"))
+    wall, ev_us, steps, warm_done = time_workload(wl, args.steps, args.warmup, use_graph=(args.launch == "graph"))
     us_per_step = wall * 1e6 / steps
     value = wl.bytes / (wall / steps) / 1e9
     kernel_us = ev_us
@@ -249,6 +289,7 @@ def main():
         "n_gpus": 1,
         "steps": steps,
         "warmup": args.warmup,
+        "warmup_steps_run": warm_done,
         "ms_per_step": round(us_per_step / 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
@@ -262,7 +303,7 @@ def main():
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "algorithmic_bytes_per_call": wl.bytes,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic_bytes(wl.name, wl.m_batch),
                      "kernel_us_avg_events": round(kernel_us, 3)},
     }
     if not args.no_cpu:
@@ -279,7 +320,7 @@ def main():
     others = {}
     for name in [n for n in args.extra.split(",") if n and n != args.workload]:
         w2 = Workload(name, device)
-        wall2, ev2, st2 = time_workload(w2, max(200, args.steps // 8), max(20, args.warmup // 4), use_graph=(args.launch == "graph"))
+        wall2, ev2, st2, _ = time_workload(w2, max(200, args.steps // 8), max(20, args.warmup // 4), use_graph=(args.launch == "graph"))
         others[name] = {"workload": w2.description, "us_per_call": round(wall2 * 1e6 / st2, 3),
                         "value_GBps": round(w2.bytes / (wall2 / st2) / 1e9, 1),
                         "kernel_us_avg_events": round(ev2, 3),

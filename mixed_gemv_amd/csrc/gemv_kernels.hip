@@ -26,11 +26,9 @@ constexpr int kMaxWavesPerMfmaWorkgroup = 8;  // leaves each wave of the matrix-
 constexpr int kNumXcd = 8;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 
-// Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are the
-// ones a wave needs before it can issue its first loads; the build asks the compiler to
-// preload them into SGPRs at wave launch, which takes the kernarg fetch (a round trip to
-// memory) off the critical path of these microsecond-scale kernels.  Everything else sits in
-// GemvTail and is only needed once the k loop is under way.
+// Kernel arguments.  The first ten (four pointers and six 32-bit words) are what a wave needs
+// to address its first loads; everything else sits in GemvTail.  The kernels pull ALL of
+// them into SGPRs with one batch of scalar loads at entry (see the asm statement there).
 struct GemvTail {
   const half_t* bias;
   half_t* y;
