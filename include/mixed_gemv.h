@@ -173,6 +173,17 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
  * tests.  Process-wide. */
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
+/* Which int4 dequantiser the kernels may use.  Both produce the same bits, rn16(rn16(q*s) + z)
+ * as gemv/warp/warp_dequantizer.h:52-59:
+ *   MGEMV_DEQUANT_AUTO (default)    per wave and k step, the one-FMA form wherever every scale
+ *                                   involved is a positive fp16 below 2^-5, else the exact-integer
+ *                                   form (the route of gemv/interleaved_numeric_conversion.h:232-291
+ *                                   followed by a multiply);
+ *   MGEMV_DEQUANT_EXACT_INTEGER     always the exact-integer form.
+ * For tests and measurements.  Process-wide. */
+enum { MGEMV_DEQUANT_AUTO = 0, MGEMV_DEQUANT_EXACT_INTEGER = 1 };
+MGEMV_API int mgemv_set_dequant_form(int form);
+
 /* Reports the geometry mgemv_gemv would use: out[0] = workgroups, out[1] = threads per
  * workgroup, out[2] = k-split waves per tile, out[3] = tiles (tile groups) per workgroup,
  * out[4] = wave steps per wave, out[5] = 1 when the matrix-core path is chosen,

@@ -18,6 +18,9 @@ from .api import (  # noqa: F401
     query_launch,
     set_launch_override,
     set_matrix_core_threshold,
+    set_dequant_form,
+    DEQUANT_AUTO,
+    DEQUANT_EXACT_INTEGER,
     unpreprocess_weights,
 )
 from ._lib import LIB_PATH, MixedGemvError  # noqa: F401

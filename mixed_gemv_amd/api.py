@@ -216,6 +216,15 @@ def set_matrix_core_threshold(min_m_batch=0):
     _lib.check(_lib.lib().mgemv_set_matrix_core_threshold(int(min_m_batch)), "set_matrix_core_threshold")
 
 
+DEQUANT_AUTO = 0
+DEQUANT_EXACT_INTEGER = 1
+
+
+def set_dequant_form(form=DEQUANT_AUTO):
+    """Which int4 dequantiser the kernels may use (same bits either way); see mgemv_set_dequant_form."""
+    _lib.check(_lib.lib().mgemv_set_dequant_form(int(form)), "set_dequant_form")
+
+
 def query_launch(n_out, m_batch, k, weight_bits=4):
     out = (ctypes.c_int * 7)()
     _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), ctypes.byref(out)),

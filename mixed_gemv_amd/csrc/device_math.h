@@ -32,8 +32,8 @@ __device__ __forceinline__ half2_t splat(half_t v) { return half2_t{v, v}; }
 // magic already sit in registers; the empty asm keeps the compiler from folding them back
 // into literals (which would split the operation into v_and + v_or).
 struct ConvertRegs {
-  uint32_t mask_lo;   // 0x000f000f   nibble 0 of each 16-bit half
-  uint32_t mask_hi;   // 0x00f000f0   nibble 1 of each 16-bit half
+  uint32_t mask7;     // 0x07800780   the 4-bit field at bits 7-10 of each 16-bit half
+  uint32_t mask3;     // 0x00780078   the 4-bit field at bits 3-6 of each 16-bit half
   uint32_t magic;     // 0x64006400   fp16 1024.0 in both halves
   uint32_t sel_lo;    // v_perm selector: bytes 0,1 of a word into the low byte of each half
   uint32_t sel_hi;    // v_perm selector: bytes 2,3
@@ -41,39 +41,80 @@ struct ConvertRegs {
 
 __device__ __forceinline__ ConvertRegs make_convert_regs() {
   ConvertRegs c;
-  c.mask_lo = 0x000f000fu;
-  c.mask_hi = 0x00f000f0u;
+  c.mask7 = 0x07800780u;
+  c.mask3 = 0x00780078u;
   c.magic = 0x64006400u;
   c.sel_lo = 0x04010400u;
   c.sel_hi = 0x04030402u;
-  asm("" : "+s"(c.mask_lo));
-  asm("" : "+s"(c.mask_hi));
+  asm("" : "+s"(c.mask7));
+  asm("" : "+s"(c.mask3));
   asm("" : "+v"(c.magic));
   asm("" : "+s"(c.sel_lo));
   asm("" : "+s"(c.sel_hi));
   return c;
 }
 
-// int4: one stored word (8 biased nibbles in the order of tile_layout.h) -> 8 fp16 values,
-// exact integers in [-8, 7], as 4 packed pairs in ascending k.
-//   (w & 0x000f000f) | 0x6400_6400  is the pair (1024 + u0, 1024 + u1);  minus 1032 -> u - 8
-//   (w & 0x00f000f0) | 0x6400_6400  is the pair (1024 + 16 u2, 1024 + 16 u3);  * 1/16 - 72 -> u - 8
-// and the same on w >> 8.  All four operations are exact in fp16.  This is the bit-level
-// contract of gemv/interleaved_numeric_conversion.h:232-291 (lop3 / sub.f16x2 / fma.rn.f16x2)
-// expressed in v_and_or_b32, v_pk_add_f16 and v_pk_fma_f16.
+__device__ __forceinline__ uint32_t rotate_right_8(uint32_t w) { return __builtin_amdgcn_alignbit(w, w, 8); }
+
+// int4, general form: one stored word (8 biased 4-bit fields in the order of tile_layout.h)
+// -> 8 fp16 values, exact integers in [-8, 7], as 4 packed pairs in ascending k.
+//   (v & 0x00780078) | 0x6400_6400  is the pair (1024 + 8 u, 1024 + 8 u');  * 1/8 - 136 -> u - 8
+// for v = w >> 4, w, rotr(w, 12) and w >> 8.  Every step is exact in fp16.  This is the
+// numeric contract of gemv/interleaved_numeric_conversion.h:232-291 (lop3 / sub.f16x2 /
+// fma.rn.f16x2: biased nibble under a 1024.0 exponent, then an exact affine map) expressed
+// in v_alignbit_b32, v_and_or_b32 and v_pk_fma_f16.  (It shares no intermediate with the
+// short form below, so the compiler has nothing to hoist in front of the branch between them.)
 __device__ __forceinline__ void convert_int4_word(uint32_t w, const ConvertRegs& c, half2_t (&q)[4]) {
-  const uint32_t t = w >> 8;
-  const half2_t h0 = as_half2((w & c.mask_lo) | c.magic);
-  const half2_t h1 = as_half2((w & c.mask_hi) | c.magic);
-  const half2_t h2 = as_half2((t & c.mask_lo) | c.magic);
-  const half2_t h3 = as_half2((t & c.mask_hi) | c.magic);
-  const half2_t k1032 = splat((half_t)1032.0f);
-  const half2_t k16th = splat((half_t)0.0625f);
-  const half2_t kn72 = splat((half_t)-72.0f);
-  q[0] = h0 - k1032;
-  q[1] = __builtin_elementwise_fma(h1, k16th, kn72);
-  q[2] = h2 - k1032;
-  q[3] = __builtin_elementwise_fma(h3, k16th, kn72);
+  const half2_t h0 = as_half2(((w >> 4) & c.mask3) | c.magic);
+  const half2_t h1 = as_half2((w & c.mask3) | c.magic);
+  const half2_t h2 = as_half2((__builtin_amdgcn_alignbit(w, w, 12) & c.mask3) | c.magic);
+  const half2_t h3 = as_half2(((w >> 8) & c.mask3) | c.magic);
+  const half2_t k8th = splat((half_t)0.125f);
+  const half2_t kn136 = splat((half_t)-136.0f);
+  q[0] = __builtin_elementwise_fma(h0, k8th, kn136);
+  q[1] = __builtin_elementwise_fma(h1, k8th, kn136);
+  q[2] = __builtin_elementwise_fma(h2, k8th, kn136);
+  q[3] = __builtin_elementwise_fma(h3, k8th, kn136);
+}
+
+// int4, short form for a positive scale s below 2^-5.  A masked half-word read as fp16 IS
+// u * 2^-17 (field at bits 7-10) or u * 2^-21 (field at bits 3-6), exactly; with the scale
+// pre-multiplied by 2^17 / 2^21 (exact: s * 2^21 <= 65504) a single fused multiply-add
+//     fma(u * 2^-p, s * 2^p, -8 s)  =  rn16(u s - 8 s)  =  rn16((u - 8) * s)
+// rounds the exact product once, which is bit for bit the rn16(q * s) of
+// gemv/warp/warp_dequantizer.h:52-59; the additive zero then follows as its own rounded
+// add.  8 s is exact, and for s > 0 a zero product is +0 on both routes.  Outside
+// 0 < s < 2^-5 (large, zero, negative, NaN) the general form above is used instead.
+struct ShortFormScale {
+  half2_t s17;   // (s * 2^17, s * 2^17)
+  half2_t s21;   // (s * 2^21, s * 2^21)
+  half2_t m8s;   // (-8 s, -8 s)
+};
+
+// fp16 bit pattern of a scale for which the short form is exact: 0x0001 .. 0x27ff.
+__device__ __forceinline__ bool short_form_ok(uint32_t scale_bits) { return ((scale_bits & 0xffffu) - 1u) < 0x27ffu; }
+
+__device__ __forceinline__ ShortFormScale make_short_form_scale(half2_t s2) {
+  ShortFormScale f;
+  const half2_t a = s2 * splat((half_t)32768.0f);  // 2^17 itself is not an fp16 value
+  f.s17 = a * splat((half_t)4.0f);
+  f.s21 = f.s17 * splat((half_t)16.0f);
+  f.m8s = s2 * splat((half_t)-8.0f);
+  return f;
+}
+
+template <bool HAS_ZERO>
+__device__ __forceinline__ void dequant_int4_word_short(uint32_t w, const ConvertRegs& c, const ShortFormScale& f,
+                                                        half2_t z2, half2_t (&d)[4]) {
+  const uint32_t t = rotate_right_8(w);
+  d[0] = __builtin_elementwise_fma(as_half2(w & c.mask7), f.s17, f.m8s);
+  d[1] = __builtin_elementwise_fma(as_half2(w & c.mask3), f.s21, f.m8s);
+  d[2] = __builtin_elementwise_fma(as_half2(t & c.mask7), f.s17, f.m8s);
+  d[3] = __builtin_elementwise_fma(as_half2(t & c.mask3), f.s21, f.m8s);
+  if (HAS_ZERO) {
+#pragma unroll
+    for (int h = 0; h < 4; ++h) d[h] = d[h] + z2;
+  }
 }
 
 // int8: one stored word (4 biased bytes, natural order) -> 4 fp16 exact integers in

@@ -22,9 +22,11 @@ namespace mgemv {
 
 constexpr int kWave = 64;
 constexpr int kMaxWavesPerWorkgroup = 16;
+constexpr int kMaxWavesPerWideWorkgroup = 8;  // VALU kernel with 3-4 activation rows: 256 VGPRs per wave
 constexpr int kMaxWavesPerMfmaWorkgroup = 8;  // leaves each wave of the matrix-core kernel 256 VGPRs
 constexpr int kNumXcd = 8;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
+constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
 
 // Kernel arguments.  The first ten (four pointers and six 32-bit words) are what a wave needs
 // to address its first loads; everything else sits in GemvTail.  The kernels pull ALL of
@@ -35,7 +37,7 @@ struct GemvTail {
   int split_k;         // waves of a workgroup that share one tile (blockDim.x / 64)
   int m_batch;         // activation rows (matrix-core kernel)
   int num_groups;      // k / group_size (1 in per-column mode): extent of the scale / zero tables
-  int reserved;
+  int flags;           // kExactIntegerFormOnly or 0
   long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
 };
 
@@ -155,9 +157,6 @@ __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>
                                           int row) {
   using G = Geometry<BITS>;
 #pragma unroll
-  for (int i = 0; i < kBlocksPerUnit; ++i)
-    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c.w_voffset + i * kBlockBytes, 0, kCacheStream);
-#pragma unroll
   for (int m = 0; m < MB; ++m) {
     if constexpr (BITS == 4) {
       const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc[m], c.x_voffset, 0, kCacheDefault);
@@ -181,25 +180,37 @@ __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>
         f.z[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.zero, voffset, 0, kCacheDefault);
     }
   }
+  // The weight blocks go last: loads return in order, so block i can be consumed as soon as
+  // its own chunk is in, with only the later blocks (and the next unit) still outstanding.
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i)
+    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, c.w_voffset + i * kBlockBytes, 0, kCacheStream);
 }
 
 // One 32-bit word of block I: convert, dequantise, dot.  Lane (4 I + J) of the DPP row holds
-// the activations that pair with this word.
-template <int BITS, bool HAS_ZERO, int MB, int I, int J>
+// the activations that pair with this word.  SHORT selects the single-FMA int4 dequantiser
+// (device_math.h); the caller guarantees that every lane's scale permits it.
+template <int BITS, bool HAS_ZERO, bool SHORT, int MB, int I, int J>
 __device__ __forceinline__ void compute_word(float (&acc)[MB], uint32_t w, const uint32_t (&x)[MB][BITS == 4 ? 4 : 2],
-                                             const ConvertRegs& c, half2_t s2, half2_t z2) {
+                                             const ConvertRegs& c, half2_t s2, half2_t z2, const ShortFormScale& f) {
   constexpr int kPairs = BITS == 4 ? 4 : 2;
-  half2_t q[kPairs];
-  if constexpr (BITS == 4) convert_int4_word(w, c, q); else convert_int8_word(w, c, q);
+  half2_t d[kPairs];
+  if constexpr (BITS == 4 && SHORT) {
+    dequant_int4_word_short<HAS_ZERO>(w, c, f, z2, d);
+  } else {
+    half2_t q[kPairs];
+    if constexpr (BITS == 4) convert_int4_word(w, c, q); else convert_int8_word(w, c, q);
+#pragma unroll
+    for (int h = 0; h < kPairs; ++h) d[h] = dequant_pair<HAS_ZERO>(q[h], s2, z2);
+  }
 #pragma unroll
   for (int h = 0; h < kPairs; ++h) {
-    const half2_t d = dequant_pair<HAS_ZERO>(q[h], s2, z2);
 #pragma unroll
-    for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + J>(acc[m], x[m][h], d);
+    for (int m = 0; m < MB; ++m) dot2_row_bcast<4 * I + J>(acc[m], x[m][h], d[h]);
   }
 }
 
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, int I>
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT, int I>
 __device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
                                               const ConvertRegs& c, half2_t col_scale2) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
@@ -207,19 +218,51 @@ __device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragme
   half2_t s2 = col_scale2, z2 = half2_t{};
   if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) s2 = splat_low(f.s[gi]);
   if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
-  compute_word<BITS, kHasZero, MB, I, 0>(acc, f.w[I][0], f.x, c, s2, z2);
-  compute_word<BITS, kHasZero, MB, I, 1>(acc, f.w[I][1], f.x, c, s2, z2);
-  compute_word<BITS, kHasZero, MB, I, 2>(acc, f.w[I][2], f.x, c, s2, z2);
-  compute_word<BITS, kHasZero, MB, I, 3>(acc, f.w[I][3], f.x, c, s2, z2);
+  ShortFormScale sf{};
+  if constexpr (BITS == 4 && SHORT) sf = make_short_form_scale(s2);
+  compute_word<BITS, kHasZero, SHORT, MB, I, 0>(acc, f.w[I][0], f.x, c, s2, z2, sf);
+  compute_word<BITS, kHasZero, SHORT, MB, I, 1>(acc, f.w[I][1], f.x, c, s2, z2, sf);
+  compute_word<BITS, kHasZero, SHORT, MB, I, 2>(acc, f.w[I][2], f.x, c, s2, z2, sf);
+  compute_word<BITS, kHasZero, SHORT, MB, I, 3>(acc, f.w[I][3], f.x, c, s2, z2, sf);
 }
 
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT>
+__device__ __forceinline__ void compute_unit_form(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
+                                                  const ConvertRegs& c, half2_t col_scale2) {
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 0>(acc, f, c, col_scale2);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 1>(acc, f, c, col_scale2);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 2>(acc, f, c, col_scale2);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 3>(acc, f, c, col_scale2);
+  // The two forms meet again after this call, and the compiler may place a register copy of
+  // the accumulators at that join: make them safe to read by any instruction first.
+#pragma unroll
+  for (int m = 0; m < MB; ++m) settle_dot_chain(acc[m]);
+}
+
+// True when the scale of every lane of the wave (all groups of the unit) permits the short
+// int4 dequantiser; wave-uniform, so the choice costs one scalar branch per unit.
+template <int GROUPS_PER_RUN>
+__device__ __forceinline__ bool wave_scales_permit_short_form(const uint32_t (&scale_bits)[GROUPS_PER_RUN]) {
+  bool ok = true;
+#pragma unroll
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) ok = ok && short_form_ok(scale_bits[gi]);
+  return __builtin_amdgcn_ballot_w64(!ok) == 0;
+}
+
+// short_allowed: wave-uniform; in per-column mode it already includes the check of the
+// (loop-invariant) row scales.
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
-                                             const ConvertRegs& c, half2_t col_scale2) {
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 0>(acc, f, c, col_scale2);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 1>(acc, f, c, col_scale2);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 2>(acc, f, c, col_scale2);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, 3>(acc, f, c, col_scale2);
+                                             const ConvertRegs& c, half2_t col_scale2, bool short_allowed) {
+  if constexpr (BITS == 4) {
+    bool take_short = short_allowed;
+    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form(f.s);
+    if (take_short) {
+      compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, true>(acc, f, c, col_scale2);
+      return;
+    }
+  }
+  compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, false>(acc, f, c, col_scale2);
 }
 
 // Sum over the four k slices of a wave: lanes l, l+16, l+32, l+48 hold the same row.
@@ -244,7 +287,7 @@ __device__ __forceinline__ void store_outputs(const GemvTail& tail, bool has_bia
 // blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: tiles_per_wg * split_k * MB * 64 floats
 // (none when split_k == 1).
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
-__global__ void __launch_bounds__(kWave * kMaxWavesPerWorkgroup)
+__global__ void __launch_bounds__(kWave * (MB >= 3 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
 gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
                 uint32_t packed_steps, int workgroups, int wgs_per_xcd, uint32_t packed_group, GemvTail tail) {
   extern __shared__ float partials[];
@@ -266,7 +309,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   // load-wait pairs in front of the first weight load of these microsecond-scale kernels.
   asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
                "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
-               "s"(tail.num_groups), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
+               "s"(tail.num_groups), "s"(tail.flags), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
                "s"(tail.stride_bias), "s"(tail.stride_y));
   // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223); branch-free.
   const long long batch = blockIdx.z;
@@ -315,10 +358,15 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
     load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur, lane, row);
     half2_t col_scale = half2_t{};
-    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale = splat(p.scale[row]);
+    bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
+    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+      col_scale = splat(p.scale[row]);
+      const uint32_t bits[1] = {as_u32(col_scale)};
+      short_ok = short_ok && wave_scales_permit_short_form(bits);
+    }
     const ConvertRegs c = make_convert_regs();
     if (units == 1) {
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale, short_ok);
     } else {
       // The prefetches are unconditional: past the wave's last unit every offset is out of the
       // descriptors' range, the loads return zero without touching memory, and the compiler
@@ -328,12 +376,12 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         advance(cur);
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur, lane, row);
         __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
-        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale);
+        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale, short_ok);
         advance(cur);
         __builtin_amdgcn_sched_barrier(0);
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur, lane, row);
         __builtin_amdgcn_sched_barrier(0);
-        if (u + 1 < units) compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, col_scale);
+        if (u + 1 < units) compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, col_scale, short_ok);
         __builtin_amdgcn_sched_barrier(0);
         u += 2;
       } while (u < units);
@@ -441,10 +489,10 @@ __device__ __forceinline__ void load_weights_mfma(MfmaWeights<BITS, GROUPS_PER_R
   }
 }
 
-template <int BITS, int QOP, int GROUPS_PER_RUN>
-__device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
-                                                  const MfmaActivations<BITS>& xa, const ConvertRegs& c,
-                                                  half2_t col_scale2) {
+template <int BITS, int QOP, int GROUPS_PER_RUN, bool SHORT>
+__device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
+                                                       const MfmaActivations<BITS>& xa, const ConvertRegs& c,
+                                                       half2_t col_scale2) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i) {
@@ -453,13 +501,22 @@ __device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<
     if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) s2 = splat_low(f.s[gi]);
     if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
     if constexpr (BITS == 4) {
+      ShortFormScale sf{};
+      if constexpr (SHORT) sf = make_short_form_scale(s2);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        half2_t q[4];
-        convert_int4_word(f.w[i][j], c, q);
+        half2_t d[4];
+        if constexpr (SHORT) {
+          dequant_int4_word_short<kHasZero>(f.w[i][j], c, sf, z2, d);
+        } else {
+          half2_t q[4];
+          convert_int4_word(f.w[i][j], c, q);
+#pragma unroll
+          for (int h = 0; h < 4; ++h) d[h] = dequant_pair<kHasZero>(q[h], s2, z2);
+        }
         u32x4 a;
 #pragma unroll
-        for (int h = 0; h < 4; ++h) a[h] = as_u32(dequant_pair<kHasZero>(q[h], s2, z2));
+        for (int h = 0; h < 4; ++h) a[h] = as_u32(d[h]);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, xa.x[i][j]),
                                                      acc, 0, 0, 0);
       }
@@ -479,6 +536,21 @@ __device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<
       }
     }
   }
+}
+
+template <int BITS, int QOP, int GROUPS_PER_RUN>
+__device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
+                                                  const MfmaActivations<BITS>& xa, const ConvertRegs& c,
+                                                  half2_t col_scale2, bool short_allowed) {
+  if constexpr (BITS == 4) {
+    bool take_short = short_allowed;
+    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form(f.s);
+    if (take_short) {
+      compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, true>(acc, f, xa, c, col_scale2);
+      return;
+    }
+  }
+  compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, false>(acc, f, xa, c, col_scale2);
 }
 
 // blockDim = (64 * split_k, tiles_per_wg); each wave works on T consecutive tiles so that the
@@ -505,7 +577,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   p.tiles_per_wg = (int)(packed_group >> 24);
   asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
                "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
-               "s"(tail.m_batch), "s"(tail.num_groups), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
+               "s"(tail.m_batch), "s"(tail.num_groups), "s"(tail.flags), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
                "s"(tail.stride_bias), "s"(tail.stride_y));
   const long long batch = blockIdx.z;
   p.weights += batch * tail.stride_weights;
@@ -547,10 +619,16 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
         (uint32_t)(my_tiles - 1) * (uint32_t)tile_stride + (uint32_t)units * (uint32_t)kUnitBytes);
     const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(p.x, (uint32_t)m_batch * (uint32_t)p.k * 2u);
     half2_t col_scale[T];
+    bool short_ok[T];
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       col_scale[t] = half2_t{};
-      if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) col_scale[t] = splat(p.scale[row[t]]);
+      short_ok[t] = (tail.flags & kExactIntegerFormOnly) == 0;
+      if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+        col_scale[t] = splat(p.scale[row[t]]);
+        const uint32_t bits[1] = {as_u32(col_scale[t])};
+        short_ok[t] = short_ok[t] && wave_scales_permit_short_form(bits);
+      }
     }
     const ConvertRegs c = make_convert_regs();
     for (int u = 0; u < units; ++u) {
@@ -562,7 +640,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
                                                      ks_begin + u, lane, row[t]);  // tiles past the matrix re-read the last one; never stored
       load_activations_mfma<BITS>(xa, p, x_rsrc, ks_begin + u, lane);
 #pragma unroll
-      for (int t = 0; t < T; ++t) compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc[t], wt[t], xa, c, col_scale[t]);
+      for (int t = 0; t < T; ++t) compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc[t], wt[t], xa, c, col_scale[t], short_ok[t]);
     }
   }
 
@@ -618,49 +696,64 @@ struct DequantParams {
   const uint8_t* weights;
   const half_t* scale;
   const half_t* zero_add;
-  int n_out, k, group_size, tiles, ksteps;
+  int n_out, k, group_size, tiles, ksteps, flags;
 };
 
-// One wave per unit; writes the dequantised weights of its 16 rows x kStepK columns.
+// One wave per unit; writes the dequantised weights of its 16 rows x kStepK columns with the
+// same converters, and the same wave-uniform choice between them, as the GEMV kernels.
 template <int BITS, int QOP>
 __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, half_t* __restrict__ out) {
   using G = Geometry<BITS>;
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
   const int lane = threadIdx.x % kWave;
   const long long unit = (long long)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
-  if (unit >= (long long)p.tiles * p.ksteps) return;
+  if (unit >= (long long)p.tiles * p.ksteps) return;  // whole waves only
   const int tile = (int)(unit / p.ksteps), kstep = (int)(unit % p.ksteps);
   const int row = tile * kTileRows + lane % kTileRows;
   const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
   const ConvertRegs c = make_convert_regs();
   const uint8_t* base = p.weights + (size_t)unit * kUnitBytes + (size_t)lane * kChunkBytes;
   const int row_c = row < p.n_out ? row : p.n_out - 1;
+  uint32_t s_bits[kBlocksPerUnit];
+  half_t s[kBlocksPerUnit], z[kBlocksPerUnit];
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i) {
-    const int k0 = k_run + i * G::kChunkK;
-    const u32x4 w = *reinterpret_cast<const u32x4*>(base + i * kBlockBytes);
-    half_t s, z = (half_t)0.0f;
+    z[i] = (half_t)0.0f;
     if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
-      s = p.scale[row_c];
+      s[i] = p.scale[row_c];
     } else {
       Problem geo{};
       geo.k = p.k;
       geo.group_size = p.group_size;
-      const int idx = group_of(geo, k0) * p.n_out + row_c;
-      s = p.scale[idx];
-      if constexpr (kHasZero) z = p.zero_add[idx];
+      const int idx = group_of(geo, k_run + i * G::kChunkK) * p.n_out + row_c;
+      s[i] = p.scale[idx];
+      if constexpr (kHasZero) z[i] = p.zero_add[idx];
     }
-    const half2_t s2 = splat(s), z2 = splat(z);
+    s_bits[i] = (uint32_t)__builtin_bit_cast(uint16_t, s[i]);
+  }
+  const bool take_short =
+      BITS == 4 && (p.flags & kExactIntegerFormOnly) == 0 && wave_scales_permit_short_form(s_bits);
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) {
+    const int k0 = k_run + i * G::kChunkK;
+    const u32x4 w = *reinterpret_cast<const u32x4*>(base + i * kBlockBytes);
+    const half2_t s2 = splat(s[i]), z2 = splat(z[i]);
     if (row >= p.n_out || k0 >= p.k) continue;
     half_t* dst = out + (size_t)row * (size_t)p.k + k0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if constexpr (BITS == 4) {
-        half2_t q[4];
-        convert_int4_word(w[j], c, q);
+        half2_t d[4];
+        if (take_short) {
+          dequant_int4_word_short<kHasZero>(w[j], c, make_short_form_scale(s2), z2, d);
+        } else {
+          half2_t q[4];
+          convert_int4_word(w[j], c, q);
 #pragma unroll
-        for (int h = 0; h < 4; ++h)
-          *reinterpret_cast<half2_t*>(dst + j * 8 + h * 2) = dequant_pair<kHasZero>(q[h], s2, z2);
+          for (int h = 0; h < 4; ++h) d[h] = dequant_pair<kHasZero>(q[h], s2, z2);
+        }
+#pragma unroll
+        for (int h = 0; h < 4; ++h) *reinterpret_cast<half2_t*>(dst + j * 8 + h * 2) = d[h];
       } else {
         half2_t q[2];
         convert_int8_word(w[j], c, q);
@@ -680,6 +773,7 @@ std::atomic<int> g_override_split_k{0};
 std::atomic<int> g_override_tiles_per_wg{0};
 std::atomic<int> g_override_tiles_per_wave{0};
 std::atomic<int> g_matrix_core_min_batch{5};  // m_batch from which the matrix-core kernel is used
+std::atomic<int> g_dequant_flags{0};          // kExactIntegerFormOnly or 0
 
 inline bool use_matrix_cores(int m_batch) { return m_batch >= g_matrix_core_min_batch.load(); }
 
@@ -711,7 +805,9 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   //  * more tile groups than that: split as far as the units allow (at most 16 waves) while the
   //    launch stays under ~8k waves, and fall back to two units per wave when that still
   //    leaves >= 4096 waves (8192x8192: 10.6 us at 8 waves vs 11.2 us at 16).
-  const int max_waves = use_matrix_cores(m_batch) ? kMaxWavesPerMfmaWorkgroup : kMaxWavesPerWorkgroup;
+  const int max_waves = use_matrix_cores(m_batch) ? kMaxWavesPerMfmaWorkgroup
+                        : m_batch >= 3            ? kMaxWavesPerWideWorkgroup
+                                                  : kMaxWavesPerWorkgroup;
   int split_k;
   if (groups <= 384) {
     split_k = ksteps < 4 ? ksteps : 4;
@@ -929,6 +1025,7 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
+  g.tail.flags = g_dequant_flags.load();
   g.tail.stride_weights = stride_weights;
   g.tail.stride_x = stride_x;
   g.tail.stride_scale = stride_scale;
@@ -980,6 +1077,7 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
   p.group_size = group_size;
   p.tiles = num_tiles(n_out);
   p.ksteps = num_ksteps(k, weight_bits);
+  p.flags = g_dequant_flags.load();
   const hipError_t e = weight_bits == 4
                            ? launch_dequant<4>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream))
                            : launch_dequant<8>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream));
@@ -998,6 +1096,12 @@ int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int ti
 int mgemv_set_matrix_core_threshold(int min_m_batch) {
   if (min_m_batch < 0 || min_m_batch > MGEMV_MAX_M_BATCH + 1) return MGEMV_ERR_BATCH;
   mgemv::g_matrix_core_min_batch.store(min_m_batch == 0 ? 5 : min_m_batch);
+  return MGEMV_OK;
+}
+
+int mgemv_set_dequant_form(int form) {
+  if (form != MGEMV_DEQUANT_AUTO && form != MGEMV_DEQUANT_EXACT_INTEGER) return MGEMV_ERR_SIZE;
+  mgemv::g_dequant_flags.store(form == MGEMV_DEQUANT_EXACT_INTEGER ? mgemv::kExactIntegerFormOnly : 0);
   return MGEMV_OK;
 }
 

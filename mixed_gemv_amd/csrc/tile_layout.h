@@ -24,8 +24,16 @@
 // instructions, so the small-batch path consumes the identical buffer.
 //
 // A chunk is four 32-bit words in ascending k.  int4: a word holds 8 consecutive elements,
-// each stored biased (value + 8) in nibble position  (e % 2) * 4 + e / 2, which lets one
-// AND+OR pull a k-adjacent pair of elements into the two halves of a packed-fp16 register.
+// each stored biased (value + 8) as a 4-bit field whose least significant bit sits at bit
+// int4_field_shift(e) of the word (the field of element 5 wraps round from bit 31 to bits 0-2):
+//     e      0   1   2   3   4   5   6   7
+//     bits  7-10 23-26 3-6 19-22 15-18 31,0-2 11-14 27-30
+// The k-adjacent pair (2h, 2h+1) always lands at the SAME position of the two 16-bit halves,
+// either at bits 7-10 or at bits 3-6 of the half, directly (h = 0, 1) or after rotating the
+// word right by 8 (h = 2, 3).  Read as fp16, a half-word that is zero outside bits 0-10 has
+// the value (bits) * 2^-24 -- exponent fields 0 and 1 continue each other linearly -- so one
+// AND yields the packed pair (u * 2^-17, u' * 2^-17) or (u * 2^-21, u' * 2^-21) with no
+// integer-to-float conversion at all; the kernels fold the missing power of two into the scale.
 // int8: a word holds 4 consecutive elements in natural byte order, stored biased (value + 128).
 //
 // Rows are padded to a multiple of 16 and k to a multiple of kStepK with zero bytes; padded
@@ -81,28 +89,22 @@ MGEMV_HD size_t chunk_offset(size_t n, size_t k0, size_t ksteps, int bits) {
   return (t * ksteps + s) * (size_t)kUnitBytes + blk * (size_t)kBlockBytes + lane * (size_t)kChunkBytes;
 }
 
-// int4 word: natural nibble order (element e in bits 4e..4e+3, two's complement) ->
-// stored order (biased, element e in nibble (e%2)*4 + e/2).
-MGEMV_HD uint32_t squeeze_nibbles(uint32_t v) {  // nibbles at 0,8,16,24 -> 0,4,8,12
-  v = (v | (v >> 4)) & 0x00ff00ffu;
-  v = (v | (v >> 8)) & 0x0000ffffu;
-  return v;
-}
-MGEMV_HD uint32_t spread_nibbles(uint32_t v) {  // nibbles at 0,4,8,12 -> 0,8,16,24
-  v = (v | (v << 8)) & 0x00ff00ffu;
-  v = (v | (v << 4)) & 0x0f0f0f0fu;
-  return v;
+// int4 word: natural order (element e in bits 4e..4e+3, two's complement) <-> stored order.
+MGEMV_HD uint32_t rotl32(uint32_t v, int s) { return s ? (v << s) | (v >> (32 - s)) : v; }
+MGEMV_HD uint32_t rotr32(uint32_t v, int s) { return s ? (v >> s) | (v << (32 - s)) : v; }
+MGEMV_HD int int4_field_shift(int e) {
+  return e == 0 ? 7 : e == 1 ? 23 : e == 2 ? 3 : e == 3 ? 19 : e == 4 ? 15 : e == 5 ? 31 : e == 6 ? 11 : 27;
 }
 MGEMV_HD uint32_t encode_int4_word(uint32_t natural) {
-  uint32_t b = natural ^ 0x88888888u;  // +8 on each two's-complement nibble
-  uint32_t even = b & 0x0f0f0f0fu;
-  uint32_t odd = (b >> 4) & 0x0f0f0f0fu;
-  return squeeze_nibbles(even) | (squeeze_nibbles(odd) << 16);
+  const uint32_t b = natural ^ 0x88888888u;  // +8 on each two's-complement nibble
+  uint32_t w = 0;
+  for (int e = 0; e < 8; ++e) w |= rotl32((b >> (4 * e)) & 0xfu, int4_field_shift(e));
+  return w;
 }
 MGEMV_HD uint32_t decode_int4_word(uint32_t stored) {
-  uint32_t even = spread_nibbles(stored & 0xffffu);
-  uint32_t odd = spread_nibbles(stored >> 16);
-  return (even | (odd << 4)) ^ 0x88888888u;
+  uint32_t b = 0;
+  for (int e = 0; e < 8; ++e) b |= (rotr32(stored, int4_field_shift(e)) & 0xfu) << (4 * e);
+  return b ^ 0x88888888u;
 }
 MGEMV_HD uint32_t encode_int8_word(uint32_t natural) { return natural ^ 0x80808080u; }
 MGEMV_HD uint32_t decode_int8_word(uint32_t stored) { return stored ^ 0x80808080u; }

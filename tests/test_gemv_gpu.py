@@ -103,10 +103,66 @@ def test_converter_every_16_bit_pattern(gpu):
     assert np.array_equal(out8.cpu().numpy().view(np.uint16), want8.view(np.uint16))
 
 
+@pytest.fixture
+def exact_integer_form():
+    """Forces the kernels onto the exact-integer int4 dequantiser for the duration of a test."""
+    mg.set_dequant_form(mg.DEQUANT_EXACT_INTEGER)
+    yield
+    mg.set_dequant_form(mg.DEQUANT_AUTO)
+
+
+@pytest.mark.parametrize("cfg", [c for c in SMALL if c[3] == 4], ids=[c[0] for c in SMALL if c[3] == 4])
+def test_small_parity_exact_integer_form(gpu, exact_integer_form, cfg):
+    """The same cases with the one-FMA int4 dequantiser switched off (the default scale range of
+    these problems lies below 2^-5, so test_small_parity runs them on the one-FMA form)."""
+    tag, n_out, k, bits, qop, g, mb, bias = cfg
+    check(Problem(tag, n_out, k, bits, qop, g, m_batch=mb, bias=bias), gpu)
+
+
+def test_one_fma_form_boundaries_bit_exact(gpu):
+    """Scales at and around the limits of the one-FMA int4 dequantiser (positive, below 2^-5):
+    whole tiles inside the range take it, a tile with a single lane outside must not; all modes."""
+    special = np.array([0x0001, 0x0002, 0x03FF, 0x0400, 0x0401, 0x13FF, 0x2000, 0x27FE, 0x27FF,      # inside
+                        0x2800, 0x2801, 0x3C00, 0x7BFF, 0x0000, 0x8000, 0x8001, 0xA7FF, 0xFBFF],    # outside
+                       dtype=np.uint16)
+    n_out, g, k = 16 * special.size * 2, 128, 1024
+    groups = k // g
+    scale = np.empty((groups, n_out), dtype=np.uint16)
+    for t, bits16 in enumerate(special):                 # tile t: every lane has the special value
+        scale[:, 16 * t:16 * t + 16] = bits16
+    for t, bits16 in enumerate(special):                 # tile size+t: in range, except one lane of one group
+        scale[:, 16 * (special.size + t):16 * (special.size + t) + 16] = 0x2400
+        scale[t % groups, 16 * (special.size + t) + (5 * t) % 16] = bits16
+    q = np.tile(np.arange(-8, 8, dtype=np.int8), n_out * k // 16)
+    for qop in (SCALE_AND_ZEROS, SCALE_ONLY, PER_COLUMN):
+        prob = Problem(f"edge{qop}", n_out, k, 4, qop, g if qop != PER_COLUMN else 0)
+        prob.q, prob.w_raw = q, orc.pack_int4(q)
+        prob.scale = (scale if qop != PER_COLUMN else scale[:1]).view(np.float16).copy()
+        if qop == SCALE_AND_ZEROS:
+            zero = orc.fill_uniform_f16(groups * n_out, 5, -0.01, 0.01).reshape(groups, n_out)
+            zero[0, ::2] = np.float16(0.0)
+            zero[1, ::3] = np.float16(-0.0)
+            prob.zero_add = zero
+        for form in (mg.DEQUANT_AUTO, mg.DEQUANT_EXACT_INTEGER):
+            mg.set_dequant_form(form)
+            try:
+                got = DeviceProblem(prob, gpu).dequant().view(np.uint16)
+            finally:
+                mg.set_dequant_form(mg.DEQUANT_AUTO)
+            want = prob.oracle_dequant().view(np.uint16)
+            assert int((got != want).sum()) == 0, (qop, form)
+
+
+@pytest.mark.parametrize("form", ["auto", "exact_integer"])
 @pytest.mark.parametrize("bits", [4, 8])
-def test_dequant_every_finite_scale_bit_exact(gpu, bits):
+def test_dequant_every_finite_scale_bit_exact(gpu, bits, form, request):
     """Each (row, group) gets its own scale so that ALL finite fp16 scales (subnormals, huge
-    values, both signs) meet every weight value, with an additive zero; mul-then-add, two roundings."""
+    values, both signs) meet every weight value, with an additive zero; mul-then-add, two roundings.
+    Consecutive bit patterns sit in the same tile, so the tiles whose scales all lie in
+    0x0001..0x27ff go through the one-FMA int4 dequantiser in "auto" and every value in that
+    range is met by it."""
+    if form == "exact_integer":
+        request.getfixturevalue("exact_integer_form")
     allbits = np.arange(65536, dtype=np.uint16)
     finite = allbits[(allbits & 0x7C00) != 0x7C00]           # 63488 values
     n_out, g = 64, 64
@@ -134,8 +190,9 @@ def test_one_hot_activation_is_bit_exact_through_the_gemv_kernel(gpu):
     """y[n] == dq[n, k] bit for bit: pins the dequantiser INSIDE the GEMV kernel (not only the
     debug entry) and the lane-to-k mapping of the DPP broadcast."""
     import torch
-    for bits, k in ((4, 1024), (8, 512)):
-        prob = Problem(f"onehot{bits}", 96, k, bits, SCALE_AND_ZEROS, 64, scale_range=(1e-4, 0.02))
+    for bits, k, scale_range in ((4, 1024, (1e-4, 0.02)), (4, 1024, (0.02, 0.3)), (8, 512, (1e-4, 0.02))):
+        # int4: first range on the one-FMA dequantiser, second (scales beyond 2^-5) on the exact-integer one
+        prob = Problem(f"onehot{bits}", 96, k, bits, SCALE_AND_ZEROS, 64, scale_range=scale_range)
         dev = DeviceProblem(prob, gpu)
         dq = prob.oracle_dequant().view(np.uint16)
         for kk in list(range(0, 40)) + [63, 64, 127, 128, 255, 256, 511, k - 33, k - 1]:

@@ -17,6 +17,9 @@ W4, W8 = mg.QuantType.W4_A16, mg.QuantType.W8_A16
 COL, ROW = mg.LayoutType.kColumnMajor, mg.LayoutType.kRowMajor
 
 
+# least significant bit of the stored 4-bit field of element e of a 32-bit int4 word (wraps at 32)
+INT4_FIELD_SHIFT = (7, 23, 3, 19, 15, 31, 11, 27)
+
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(REPO, "include", "mixed_gemv.h")).read()
     declared = set(re.findall(r"MGEMV_API\s+[\w\s\*]+?\b(mgemv_\w+)\s*\(", header))
@@ -79,8 +82,11 @@ def test_preprocess_layout_closed_form_and_round_trip(bits, n_out, k):
                 w = int(words[j])
                 if bits == 4:
                     for e in range(8):
-                        pos = (e % 2) * 4 + e // 2           # pair (e, e+1) sits in the two 16-bit halves
-                        assert ((w >> (4 * pos)) & 0xF) == vals[8 * j + e] + 8
+                        # pair (e, e+1) sits at the same bits of the two 16-bit halves: bits 7-10 or 3-6,
+                        # directly (e < 4) or after an 8-bit right rotation (e >= 4)
+                        shift = INT4_FIELD_SHIFT[e]
+                        rot = ((w >> shift) | (w << (32 - shift))) & 0xFFFFFFFF
+                        assert (rot & 0xF) == vals[8 * j + e] + 8
                 else:
                     for e in range(4):
                         assert ((w >> (8 * e)) & 0xFF) == vals[4 * j + e] + 128
@@ -89,12 +95,30 @@ def test_preprocess_layout_closed_form_and_round_trip(bits, n_out, k):
     assert np.array_equal(back, raw)
 
 
+def test_int4_field_positions_tile_the_word():
+    # the eight 4-bit fields cover each of the 32 bits exactly once, and the two elements of a
+    # k-adjacent pair sit 16 bits apart
+    covered = np.zeros(32, dtype=int)
+    for e, shift in enumerate(INT4_FIELD_SHIFT):
+        for b in range(4):
+            covered[(shift + b) % 32] += 1
+        if e % 2:
+            assert shift == INT4_FIELD_SHIFT[e - 1] + 16
+    assert (covered == 1).all()
+    # after the rotation that the kernels apply, every field sits at bits 7-10 or 3-6 of a half-word
+    for e, shift in enumerate(INT4_FIELD_SHIFT):
+        pos = (shift - (8 if e >= 4 else 0)) % 32
+        assert pos % 16 in (7, 3)
+
+
 def test_preprocess_is_a_bijection_on_nibbles():
     n_out, k = 32, 1024
     # every nibble distinct-ish: use a counter pattern so that a collision or a dropped chunk shows
     raw = (np.arange(n_out * k // 2, dtype=np.uint32) * 2654435761 >> 7).astype(np.uint8)
     pre = mg.MixedGemvWeightPreprocessor.run(raw, (k, n_out), COL, W4)
-    assert np.array_equal(np.sort(mg.SubBytePacker.unpack(pre)), np.sort(mg.SubBytePacker.unpack(raw ^ 0x88).astype(np.int8)))
+    words = pre.view(np.uint32).astype(np.uint64)
+    fields = np.concatenate([(((words >> s) | (words << (32 - s))) & 0xF) for s in INT4_FIELD_SHIFT]).astype(np.int8)
+    assert np.array_equal(np.sort(fields), np.sort(mg.SubBytePacker.unpack(raw ^ 0x88).astype(np.int8) & 0xF))
     assert np.array_equal(mg.unpreprocess_weights(pre, (k, n_out), W4), raw)
 
 
