@@ -162,11 +162,14 @@ MGEMV_API int mgemv_dequantize(const void *weights, const uint16_t *scale, const
                                uint16_t *out, int n_out, int k, int group_size, int quant_op, int weight_bits,
                                void *stream);
 
-/* Launch geometry override for tuning and tests: k-split waves per tile, tiles (tile groups)
- * per workgroup, and tiles handled by one wave of the matrix-core kernel (1, 2 or 4); 0
- * restores the built-in heuristic for that knob.  Process-wide.  These are the counterparts of
- * the reference's compile-time ThreadBlockShape / WarpShape choices (mixed_gemv_test.cu:67-70). */
-MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave);
+/* Launch geometry override for tuning and tests: k-split waves per tile, tile sequences per
+ * workgroup, tiles handled by one wave of the matrix-core kernel (1, 2 or 4), and the largest
+ * number of workgroups of the VALU kernel (with fewer workgroups than tiles every wave walks
+ * several consecutive tiles, one after the other); 0 restores the built-in heuristic for that
+ * knob.  Process-wide.  These are the counterparts of the reference's compile-time
+ * ThreadBlockShape / WarpShape choices (mixed_gemv_test.cu:67-70). */
+MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave,
+                                        int max_workgroups);
 
 /* Smallest m_batch served by the matrix-core kernel instead of the VALU kernel (built-in
  * default 5; 0 restores it; 17 keeps every batch size on the VALU kernel).  For tuning and
@@ -185,10 +188,11 @@ enum { MGEMV_DEQUANT_AUTO = 0, MGEMV_DEQUANT_EXACT_INTEGER = 1 };
 MGEMV_API int mgemv_set_dequant_form(int form);
 
 /* Reports the geometry mgemv_gemv would use: out[0] = workgroups, out[1] = threads per
- * workgroup, out[2] = k-split waves per tile, out[3] = tiles (tile groups) per workgroup,
- * out[4] = wave steps per wave, out[5] = 1 when the matrix-core path is chosen,
- * out[6] = tiles per wave. */
-MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[7]);
+ * workgroup, out[2] = k-split waves per tile, out[3] = tile sequences per workgroup,
+ * out[4] = k steps per wave and tile, out[5] = 1 when the matrix-core path is chosen,
+ * out[6] = tiles per wave (matrix-core path), out[7] = most tiles a wave walks one after the
+ * other (VALU path). */
+MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8]);
 
 #ifdef __cplusplus
 }

@@ -28,10 +28,10 @@ SIGNATURES = {
     "mgemv_gemv_batched": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 7
                            + [_c.c_int64] * 5 + [_vp]),
     "mgemv_dequantize": (_c.c_int, [_vp, _u16p, _u16p, _u16p] + [_c.c_int] * 5 + [_vp]),
-    "mgemv_set_launch_override": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int]),
+    "mgemv_set_launch_override": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int, _c.c_int]),
     "mgemv_set_matrix_core_threshold": (_c.c_int, [_c.c_int]),
     "mgemv_set_dequant_form": (_c.c_int, [_c.c_int]),
-    "mgemv_query_launch": (_c.c_int, [_c.c_int] * 4 + [_c.POINTER(_c.c_int * 7)]),
+    "mgemv_query_launch": (_c.c_int, [_c.c_int] * 4 + [_c.POINTER(_c.c_int * 8)]),
 }
 
 _lib = None

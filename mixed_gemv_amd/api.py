@@ -207,9 +207,9 @@ def dequantize(ptr_A, ptr_scale, ptr_zero_point, ptr_out, M, K, group_size,
     _lib.check(st, "dequantize")
 
 
-def set_launch_override(split_k_waves=0, tiles_per_workgroup=0, tiles_per_wave=0):
-    _lib.check(_lib.lib().mgemv_set_launch_override(int(split_k_waves), int(tiles_per_workgroup), int(tiles_per_wave)),
-               "set_launch_override")
+def set_launch_override(split_k_waves=0, tiles_per_workgroup=0, tiles_per_wave=0, max_workgroups=0):
+    _lib.check(_lib.lib().mgemv_set_launch_override(int(split_k_waves), int(tiles_per_workgroup), int(tiles_per_wave),
+                                                    int(max_workgroups)), "set_launch_override")
 
 
 def set_matrix_core_threshold(min_m_batch=0):
@@ -226,8 +226,9 @@ def set_dequant_form(form=DEQUANT_AUTO):
 
 
 def query_launch(n_out, m_batch, k, weight_bits=4):
-    out = (ctypes.c_int * 7)()
+    out = (ctypes.c_int * 8)()
     _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), ctypes.byref(out)),
                "query_launch")
-    keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave")
+    keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave",
+            "tiles_in_sequence")
     return dict(zip(keys, list(out)))

@@ -95,55 +95,92 @@ __device__ __forceinline__ half2_t splat_low(uint32_t bits) {
   return half2_t{h, h};
 }
 
-// Where a lane reads for the current unit.  Everything that varies along k sits in the VGPR
-// offset of the buffer loads (the part of the address that the hardware bounds-checks), so
-// reads past k or past the last group return zero instead of touching foreign memory.
+// Where a lane reads for the current unit.  Everything that varies from unit to unit sits in
+// the VGPR offset of the buffer loads (the part of the address that the hardware
+// bounds-checks), so reads past the wave's last unit return zero instead of touching foreign
+// memory.
 //
-// GROUPS_PER_RUN 1 or 2 ("regular"): the group size divides the k step, so a lane's scale /
-// zero offset just advances by a constant per unit.  GROUPS_PER_RUN 4 ("generic", any group
-// size that is a multiple of 32): one lookup per block with an integer division.
+// GROUPS_PER_RUN 1 or 2 ("regular"): the group size divides the k step (or there is a single
+// group, the per-column mode), so a lane's scale / zero offset advances by a constant per
+// unit.  GROUPS_PER_RUN 4 ("generic", any group size that is a multiple of 32): one lookup
+// per block with an integer division.
 template <int BITS, int GROUPS_PER_RUN>
 struct WaveCursor {
   int w_voffset;                   // byte offset of this lane's chunk of block 0 inside the wave's weight range
   int x_voffset;                   // byte offset of this lane's activations
   int sz_voffset[GROUPS_PER_RUN];  // regular: byte offset of this lane's scale / zero
   int k_run;                       // generic: first reduction index of the lane's run
-  int sz_stride;                   // regular: bytes per k step in the scale / zero tables
+  int row;                         // generic: this lane's row (not clamped; padded rows are never stored)
+};
+
+// A wave walks the same k range of several consecutive tiles, one after the other, as ONE
+// stream of units: these are the (wave-uniform) strides of that walk.
+struct TileWalk {
+  int units;      // units per tile for this wave
+  int left;       // units of the current tile not yet addressed
+  int w_jump;     // from the last unit of a tile to the first unit of the next tile, bytes
+  int x_back;     // activations: back to the start of the k range, bytes
+  int k_back;     // the same in reduction elements
+  int sz_stride;  // regular: bytes per k step in the scale / zero tables
+  int sz_jump;    // regular: from the last unit of a tile to the first of the next (16 rows on)
 };
 
 template <int BITS, int GROUPS_PER_RUN>
-__device__ __forceinline__ WaveCursor<BITS, GROUPS_PER_RUN> make_cursor(const Problem& p, int ks_begin, int lane, int row) {
+__device__ __forceinline__ WaveCursor<BITS, GROUPS_PER_RUN> make_cursor(const Problem& p, bool per_column, int ks_begin,
+                                                                       int units, int lane, int row, TileWalk& walk) {
   using G = Geometry<BITS>;
   WaveCursor<BITS, GROUPS_PER_RUN> c;
   c.w_voffset = lane * kChunkBytes;
   c.x_voffset = ks_begin * (G::kStepK * 2) + lane * (BITS == 4 ? 16 : 8);
   c.k_run = ks_begin * G::kStepK + (lane / kTileRows) * G::kRunK;
+  c.row = row;
+  walk.units = units;
+  walk.left = units;
+  walk.w_jump = (p.ksteps - units + 1) * kUnitBytes;
+  walk.x_back = (units - 1) * (G::kStepK * 2);
+  walk.k_back = (units - 1) * G::kStepK;
+  walk.sz_stride = 0;
   if constexpr (GROUPS_PER_RUN != 4) {
-    // Regular modes: the group size divides the k step, hence is a power of two; no divisions.
-    const int shift = __builtin_ctz((unsigned)p.group_size);
-    const int groups_per_step = G::kStepK >> shift;
-    c.sz_stride = groups_per_step * p.n_out * 2;
+    if (per_column) {
 #pragma unroll
-    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
-      const int k_local = (lane / kTileRows) * G::kRunK + gi * (G::kRunK / GROUPS_PER_RUN);
-      c.sz_voffset[gi] = ((ks_begin * groups_per_step + (k_local >> shift)) * p.n_out + row) * 2;
+      for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) c.sz_voffset[gi] = row * 2;
+    } else {
+      // Regular modes: the group size divides the k step, hence is a power of two; no divisions.
+      const int shift = __builtin_ctz((unsigned)p.group_size);
+      const int groups_per_step = G::kStepK >> shift;
+      walk.sz_stride = groups_per_step * p.n_out * 2;
+#pragma unroll
+      for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
+        const int k_local = (lane / kTileRows) * G::kRunK + gi * (G::kRunK / GROUPS_PER_RUN);
+        c.sz_voffset[gi] = ((ks_begin * groups_per_step + (k_local >> shift)) * p.n_out + row) * 2;
+      }
     }
   } else {
-    c.sz_stride = 0;
 #pragma unroll
     for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) c.sz_voffset[gi] = 0;
   }
+  walk.sz_jump = kTileRows * 2 - (units - 1) * walk.sz_stride;
   return c;
 }
 
+// To the next unit of the stream: the next k step of the same tile, or the first unit of the
+// next tile.
 template <int BITS, int GROUPS_PER_RUN>
-__device__ __forceinline__ void advance(WaveCursor<BITS, GROUPS_PER_RUN>& c) {
+__device__ __forceinline__ void advance(WaveCursor<BITS, GROUPS_PER_RUN>& c, TileWalk& walk) {
   using G = Geometry<BITS>;
-  c.w_voffset += kUnitBytes;
-  c.x_voffset += G::kStepK * 2;
-  c.k_run += G::kStepK;
+  walk.left -= 1;
+  const bool wrap = walk.left == 0;
+  c.w_voffset += wrap ? walk.w_jump : kUnitBytes;
+  c.x_voffset += wrap ? -walk.x_back : G::kStepK * 2;
+  if constexpr (GROUPS_PER_RUN == 4) {
+    c.k_run += wrap ? -walk.k_back : G::kStepK;
+    c.row += wrap ? kTileRows : 0;
+  } else {
+    const int step = wrap ? walk.sz_jump : walk.sz_stride;
 #pragma unroll
-  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) c.sz_voffset[gi] += c.sz_stride;
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) c.sz_voffset[gi] += step;
+  }
+  walk.left = wrap ? walk.units : walk.left;
 }
 
 struct ScaleTables {
@@ -153,8 +190,7 @@ struct ScaleTables {
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f, const Problem& p,
                                           __amdgpu_buffer_rsrc_t w_rsrc, const __amdgpu_buffer_rsrc_t (&x_rsrc)[MB],
-                                          const ScaleTables& tables, const WaveCursor<BITS, GROUPS_PER_RUN>& c, int lane,
-                                          int row) {
+                                          const ScaleTables& tables, const WaveCursor<BITS, GROUPS_PER_RUN>& c) {
   using G = Geometry<BITS>;
 #pragma unroll
   for (int m = 0; m < MB; ++m) {
@@ -166,19 +202,17 @@ __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>
       f.x[m][0] = v[0]; f.x[m][1] = v[1];
     }
   }
-  if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) {
 #pragma unroll
-    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
-      int voffset;
-      if constexpr (GROUPS_PER_RUN == 4) {
-        voffset = (group_of(p, c.k_run + gi * G::kChunkK) * p.n_out + row) * 2;
-      } else {
-        voffset = c.sz_voffset[gi];
-      }
-      f.s[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.scale, voffset, 0, kCacheDefault);
-      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS)
-        f.z[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.zero, voffset, 0, kCacheDefault);
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
+    int voffset;
+    if constexpr (GROUPS_PER_RUN == 4) {
+      voffset = (group_of(p, c.k_run + gi * G::kChunkK) * p.n_out + c.row) * 2;
+    } else {
+      voffset = c.sz_voffset[gi];
     }
+    f.s[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.scale, voffset, 0, kCacheDefault);
+    if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS)
+      f.z[gi] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(tables.zero, voffset, 0, kCacheDefault);
   }
   // The weight blocks go last: loads return in order, so block i can be consumed as soon as
   // its own chunk is in, with only the later blocks (and the next unit) still outstanding.
@@ -212,11 +246,11 @@ __device__ __forceinline__ void compute_word(float (&acc)[MB], uint32_t w, const
 
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT, int I>
 __device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
-                                              const ConvertRegs& c, half2_t col_scale2) {
+                                              const ConvertRegs& c) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
   constexpr int gi = I * GROUPS_PER_RUN / kBlocksPerUnit;
-  half2_t s2 = col_scale2, z2 = half2_t{};
-  if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) s2 = splat_low(f.s[gi]);
+  const half2_t s2 = splat_low(f.s[gi]);
+  half2_t z2 = half2_t{};
   if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
   ShortFormScale sf{};
   if constexpr (BITS == 4 && SHORT) sf = make_short_form_scale(s2);
@@ -228,11 +262,11 @@ __device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragme
 
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT>
 __device__ __forceinline__ void compute_unit_form(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
-                                                  const ConvertRegs& c, half2_t col_scale2) {
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 0>(acc, f, c, col_scale2);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 1>(acc, f, c, col_scale2);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 2>(acc, f, c, col_scale2);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 3>(acc, f, c, col_scale2);
+                                                  const ConvertRegs& c) {
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 0>(acc, f, c);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 1>(acc, f, c);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 2>(acc, f, c);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 3>(acc, f, c);
   // The two forms meet again after this call, and the compiler may place a register copy of
   // the accumulators at that join: make them safe to read by any instruction first.
 #pragma unroll
@@ -249,20 +283,17 @@ __device__ __forceinline__ bool wave_scales_permit_short_form(const uint32_t (&s
   return __builtin_amdgcn_ballot_w64(!ok) == 0;
 }
 
-// short_allowed: wave-uniform; in per-column mode it already includes the check of the
-// (loop-invariant) row scales.
+// short_allowed: wave-uniform.
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
-                                             const ConvertRegs& c, half2_t col_scale2, bool short_allowed) {
+                                             const ConvertRegs& c, bool short_allowed) {
   if constexpr (BITS == 4) {
-    bool take_short = short_allowed;
-    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form(f.s);
-    if (take_short) {
-      compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, true>(acc, f, c, col_scale2);
+    if (short_allowed && wave_scales_permit_short_form(f.s)) {
+      compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, true>(acc, f, c);
       return;
     }
   }
-  compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, false>(acc, f, c, col_scale2);
+  compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, false>(acc, f, c);
 }
 
 // Sum over the four k slices of a wave: lanes l, l+16, l+32, l+48 hold the same row.
@@ -284,8 +315,25 @@ __device__ __forceinline__ void store_outputs(const GemvTail& tail, bool has_bia
   }
 }
 
-// blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: tiles_per_wg * split_k * MB * 64 floats
-// (none when split_k == 1).
+// A wave has computed the last unit of a tile: hand the tile's partial sums on and start afresh.
+// split_k == 1: the wave owns the whole reduction, so it stores the outputs itself (no LDS, no
+// barrier); otherwise the 64 per-lane sums go to the wave's LDS slot for that tile.
+template <int MB>
+__device__ __forceinline__ void finish_tile(float (&acc)[MB], const GemvTail& tail, bool has_bias, int n_out, int tile,
+                                            int lane, int split_k, float* slot) {
+  if (split_k == 1) {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) store_outputs(tail, has_bias, n_out, m, tile, lane, reduce_k_slices(acc[m]));
+  } else {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) slot[m * kWave] = acc[m];
+  }
+#pragma unroll
+  for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+}
+
+// blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: ceil(tiles / sequences) * tiles_per_wg *
+// split_k * MB * 64 floats (none when split_k == 1).
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
 __global__ void __launch_bounds__(kWave * (MB >= 3 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
 gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
@@ -326,23 +374,29 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
 
   const int lane = threadIdx.x % kWave;
   const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // position along k
-  const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);         // tile within the workgroup
-  const int tile = wg * p.tiles_per_wg + ty;
+  const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);         // tile sequence within the workgroup
+  const int split_k = tail.split_k;
   const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
-  const int row_raw = tile * kTileRows + lane % kTileRows;
-  const int row = row_raw < p.n_out ? row_raw : p.n_out - 1;  // clamp padded rows (never stored)
-
-  float acc[MB];
-#pragma unroll
-  for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+  // The tiles are dealt out evenly, in contiguous runs, to the (workgroups x tiles_per_wg) tile
+  // sequences of the launch; the split_k waves of a sequence walk its tiles together, each on
+  // its own part of k.
+  const long long sequences = (long long)p.workgroups * p.tiles_per_wg;
+  const long long seq = (long long)wg * p.tiles_per_wg + ty;
+  const int tile_begin = (int)(seq * tiles / sequences);
+  const int my_tiles = (int)((seq + 1) * tiles / sequences) - tile_begin;
 
   const int ks_begin = kw * p.steps_per_wave;
   const int ks_end = min(ks_begin + p.steps_per_wave, p.ksteps);
-  if (tile < tiles && ks_begin < ks_end) {
-    const int units = ks_end - ks_begin;
+  const int units = ks_end > ks_begin ? ks_end - ks_begin : 0;
+  const int park_stride = p.tiles_per_wg * split_k * MB * kWave;  // floats between consecutive tiles of a sequence
+  float* const park = partials + (ty * split_k + kw) * MB * kWave + lane;
+
+  if (my_tiles > 0 && units > 0) {
+    const int total = my_tiles * units;
+    const int tile_stride = p.ksteps * kUnitBytes;
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
-        p.weights + ((size_t)tile * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
-        (uint32_t)units * (uint32_t)kUnitBytes);
+        p.weights + ((size_t)tile_begin * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
+        (uint32_t)(my_tiles - 1) * (uint32_t)tile_stride + (uint32_t)units * (uint32_t)kUnitBytes);
     __amdgpu_buffer_rsrc_t x_rsrc[MB];
 #pragma unroll
     for (int m = 0; m < MB; ++m) x_rsrc[m] = make_rsrc(p.x + (size_t)m * (size_t)p.k, (uint32_t)p.k * 2u);
@@ -351,65 +405,69 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     const uint32_t table_bytes = (uint32_t)tail.num_groups * (uint32_t)p.n_out * 2u;
     tables.scale = make_rsrc(p.scale, table_bytes);
     tables.zero = make_rsrc(p.zero_add, QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? table_bytes : 0u);
-    WaveCursor<BITS, GROUPS_PER_RUN> cur = make_cursor<BITS, GROUPS_PER_RUN>(p, ks_begin, lane, row);
+    TileWalk walk;
+    WaveCursor<BITS, GROUPS_PER_RUN> cur = make_cursor<BITS, GROUPS_PER_RUN>(
+        p, QOP == MGEMV_PER_COLUMN_SCALE_ONLY, ks_begin, units, lane, tile_begin * kTileRows + lane % kTileRows, walk);
+
+    float acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
+    int tile = tile_begin;   // tile whose units are being computed
+    int pending = units;     // units of that tile still to compute
+    float* slot = park;
 
     // Two fragments in flight: the loads of unit u+1 are issued before unit u is computed, so
     // a wave that is waiting for its turn on the VALU still has memory requests outstanding.
+    // The prefetches are unconditional: past the wave's last unit every weight offset is out of
+    // the descriptor's range, the loads return zero without touching memory, and the compiler
+    // can count outstanding loads exactly instead of draining them all before each use.
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
-    load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur, lane, row);
-    half2_t col_scale = half2_t{};
-    bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
-    if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
-      col_scale = splat(p.scale[row]);
-      const uint32_t bits[1] = {as_u32(col_scale)};
-      short_ok = short_ok && wave_scales_permit_short_form(bits);
-    }
+    load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
+    const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
     const ConvertRegs c = make_convert_regs();
-    if (units == 1) {
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale, short_ok);
-    } else {
-      // The prefetches are unconditional: past the wave's last unit every offset is out of the
-      // descriptors' range, the loads return zero without touching memory, and the compiler
-      // can count outstanding loads exactly instead of draining them all before each use.
-      int u = 0;
-      do {
-        advance(cur);
-        load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur, lane, row);
-        __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
-        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, col_scale, short_ok);
-        advance(cur);
-        __builtin_amdgcn_sched_barrier(0);
-        load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur, lane, row);
-        __builtin_amdgcn_sched_barrier(0);
-        if (u + 1 < units) compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, col_scale, short_ok);
-        __builtin_amdgcn_sched_barrier(0);
-        u += 2;
-      } while (u < units);
-    }
+    int u = 0;
+    do {
+      advance(cur, walk);
+      load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
+      __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, short_ok);
+      if (--pending == 0) {
+        finish_tile<MB>(acc, tail, has_bias, p.n_out, tile, lane, split_k, slot);
+        ++tile; slot += park_stride; pending = units;
+      }
+      advance(cur, walk);
+      __builtin_amdgcn_sched_barrier(0);
+      load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
+      __builtin_amdgcn_sched_barrier(0);
+      if (u + 1 < total) {
+        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, short_ok);
+        if (--pending == 0) {
+          finish_tile<MB>(acc, tail, has_bias, p.n_out, tile, lane, split_k, slot);
+          ++tile; slot += park_stride; pending = units;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      u += 2;
+    } while (u < total);
+  } else if (split_k > 1) {
+    // A wave without work (cannot happen with the launch geometry the host computes) still
+    // owes zeros to the combine below.
+    for (int j = 0; j < my_tiles; ++j) {
 #pragma unroll
-    for (int m = 0; m < MB; ++m) settle_dot_chain(acc[m]);
+      for (int m = 0; m < MB; ++m) park[j * park_stride + m * kWave] = 0.0f;
+    }
   }
 
-  const int split_k = tail.split_k;
-  if (split_k == 1) {
-    // One wave owns the whole reduction of its tile: no LDS, no barrier.
-    if (tile < tiles) {
-#pragma unroll
-      for (int m = 0; m < MB; ++m) store_outputs(tail, has_bias, p.n_out, m, tile, lane, reduce_k_slices(acc[m]));
-    }
-    return;
-  }
+  if (split_k == 1) return;  // every tile was stored by the wave that owns it
 
-  // Split-K combine (gemv/threadblock/accumulator_combine.h:269-329): every wave parks its 64
-  // per-lane partial sums in LDS; after one barrier, wave kw of each tile sums activation rows
-  // m = kw, kw + split_k, ... over the waves in ascending order, then over the four k slices.
-  const int slot = (ty * split_k + kw) * MB;
-#pragma unroll
-  for (int m = 0; m < MB; ++m) partials[(slot + m) * kWave + lane] = acc[m];
+  // Split-K combine (gemv/threadblock/accumulator_combine.h:269-329): every wave has parked
+  // its 64 per-lane partial sums of each tile in LDS; after ONE barrier the (tile, activation
+  // row) pairs of the sequence are dealt out to its waves, each summing a pair over the waves
+  // in ascending order, then over the four k slices.
   __syncthreads();
-  if (tile >= tiles) return;
-  for (int m = kw; m < MB; m += split_k) {
-    const float* part = partials + (ty * split_k * MB + m) * kWave + lane;
+  for (int item = kw; item < my_tiles * MB; item += split_k) {
+    const int j = item / MB, m = item % MB;
+    const float* part = partials + j * park_stride + (ty * split_k * MB + m) * kWave + lane;
     float sum = 0.0f;
     int w = 0;
     for (; w + 4 <= split_k; w += 4) {
@@ -418,7 +476,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       sum = (((sum + a0) + a1) + a2) + a3;
     }
     for (; w < split_k; ++w) sum += part[w * MB * kWave];
-    store_outputs(tail, has_bias, p.n_out, m, tile, lane, reduce_k_slices(sum));
+    store_outputs(tail, has_bias, p.n_out, m, tile_begin + j, lane, reduce_k_slices(sum));
   }
 }
 
@@ -772,6 +830,7 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, 
 std::atomic<int> g_override_split_k{0};
 std::atomic<int> g_override_tiles_per_wg{0};
 std::atomic<int> g_override_tiles_per_wave{0};
+std::atomic<int> g_override_workgroups{0};
 std::atomic<int> g_matrix_core_min_batch{5};  // m_batch from which the matrix-core kernel is used
 std::atomic<int> g_dequant_flags{0};          // kExactIntegerFormOnly or 0
 
@@ -780,6 +839,7 @@ inline bool use_matrix_cores(int m_batch) { return m_batch >= g_matrix_core_min_
 struct LaunchPlan {
   int split_k, tiles_per_wg, steps_per_wave, workgroups, wgs_per_xcd, threads;
   int tiles_per_wave;  // 1 on the VALU path; 1, 2 or 4 on the matrix-core path
+  int tiles_in_sequence;  // VALU path: most tiles any wave walks one after the other
 };
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -833,6 +893,22 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   lp.tiles_per_wg = tiles_per_wg;
   lp.steps_per_wave = steps;
   lp.workgroups = ceil_div(groups, tiles_per_wg);
+  lp.tiles_in_sequence = 1;
+  if (!use_matrix_cores(m_batch)) {
+    // VALU path: fewer workgroups than tile groups means every wave walks several tiles.
+    const int ov_wg = g_override_workgroups.load();
+    int cap = ov_wg > 0 ? ov_wg : lp.workgroups;
+    if (cap < lp.workgroups) lp.workgroups = cap;
+    const int rows = m_batch < kMaxValuBatch ? m_batch : kMaxValuBatch;
+    auto seq_tiles = [&]() { return ceil_div(tiles, lp.workgroups * tiles_per_wg); };
+    // limits: a wave's weight range is addressed with 32-bit offsets; the combine parks
+    // tiles x waves x rows x 64 floats in LDS
+    while (lp.workgroups < ceil_div(groups, tiles_per_wg) &&
+           ((long long)seq_tiles() * ksteps * kUnitBytes >= (1ll << 31) ||
+            (split_k > 1 && (long long)seq_tiles() * tiles_per_wg * split_k * rows * kWave * 4 > 64 * 1024)))
+      lp.workgroups = lp.workgroups * 2 < ceil_div(groups, tiles_per_wg) ? lp.workgroups * 2 : ceil_div(groups, tiles_per_wg);
+    lp.tiles_in_sequence = seq_tiles();
+  }
   lp.wgs_per_xcd = ceil_div(lp.workgroups, kNumXcd);
   lp.threads = kWave * split_k * tiles_per_wg;
   lp.tiles_per_wave = tiles_per_wave;
@@ -1049,7 +1125,8 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
     const int mb = m_batch - m0 < kMaxValuBatch ? m_batch - m0 : kMaxValuBatch;
     g.x = reinterpret_cast<const half_t*>(x) + (size_t)m0 * (size_t)k;
     g.tail.y = reinterpret_cast<half_t*>(y) + (size_t)m0 * (size_t)n_out;
-    g.lds = g.plan.split_k == 1 ? 0 : (size_t)g.plan.tiles_per_wg * g.plan.split_k * mb * kWave * sizeof(float);
+    g.lds = g.plan.split_k == 1 ? 0
+                                : (size_t)g.plan.tiles_in_sequence * g.plan.tiles_per_wg * g.plan.split_k * mb * kWave * sizeof(float);
     if (launch_gemv(g, weight_bits, quant_op, mb, gpr) != hipSuccess) return MGEMV_ERR_LAUNCH;
   }
   return MGEMV_OK;
@@ -1084,12 +1161,13 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
   return e == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
 }
 
-int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave) {
-  if (split_k_waves < 0 || tiles_per_workgroup < 0 || tiles_per_wave < 0) return MGEMV_ERR_SIZE;
+int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave, int max_workgroups) {
+  if (split_k_waves < 0 || tiles_per_workgroup < 0 || tiles_per_wave < 0 || max_workgroups < 0) return MGEMV_ERR_SIZE;
   if (tiles_per_wave != 0 && tiles_per_wave != 1 && tiles_per_wave != 2 && tiles_per_wave != 4) return MGEMV_ERR_SIZE;
   mgemv::g_override_split_k.store(split_k_waves);
   mgemv::g_override_tiles_per_wg.store(tiles_per_workgroup);
   mgemv::g_override_tiles_per_wave.store(tiles_per_wave);
+  mgemv::g_override_workgroups.store(max_workgroups);
   return MGEMV_OK;
 }
 
@@ -1105,7 +1183,7 @@ int mgemv_set_dequant_form(int form) {
   return MGEMV_OK;
 }
 
-int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[7]) {
+int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8]) {
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
   if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
@@ -1118,6 +1196,7 @@ int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[7
   out[4] = lp.steps_per_wave;
   out[5] = mgemv::use_matrix_cores(m_batch) ? 1 : 0;
   out[6] = lp.tiles_per_wave;
+  out[7] = lp.tiles_in_sequence;
   return MGEMV_OK;
 }
 

@@ -221,19 +221,23 @@ def test_split_k_invariance_and_determinism(gpu):
     ref = prob.oracle_gemv(threads=16)
     results = {}
     try:
-        for sk, tw in ((1, 1), (1, 4), (2, 2), (3, 1), (4, 4), (8, 2), (16, 1)):
-            mg.set_launch_override(sk, tw, 0)
+        # (k-split waves, tile sequences per workgroup, workgroup cap): with a cap below the 12
+        # tiles every wave walks several tiles in a row
+        for sk, tw, cap in ((1, 1, 0), (1, 4, 0), (2, 2, 0), (3, 1, 0), (4, 4, 0), (8, 2, 0), (16, 1, 0),
+                            (1, 1, 5), (4, 1, 5), (4, 2, 2), (2, 1, 1), (16, 1, 8), (1, 1, 1)):
+            mg.set_launch_override(sk, tw, 0, cap)
             a = dev.run().copy()
             b = dev.run().copy()
             assert np.array_equal(a.view(np.uint16), b.view(np.uint16)), "same launch geometry must be bit-reproducible"
             _, rel, _ = error_report(a, ref)
-            assert rel <= REL_TOL, (sk, tw, rel)
-            results[(sk, tw)] = a
+            assert rel <= REL_TOL, (sk, tw, cap, rel)
+            results[(sk, tw, cap)] = a
     finally:
-        mg.set_launch_override(0, 0, 0)
-    # different tilings of the workgroup over the same k split add in the same order
-    base = results[(1, 1)]
-    assert np.array_equal(base.view(np.uint16), results[(1, 4)].view(np.uint16))
+        mg.set_launch_override(0, 0, 0, 0)
+    # different arrangements of the tiles over workgroups and waves add in the same order
+    for same in (((1, 1, 0), (1, 4, 0), (1, 1, 5), (1, 1, 1)), ((4, 4, 0), (4, 1, 5)), ((16, 1, 0), (16, 1, 8))):
+        for other in same[1:]:
+            assert np.array_equal(results[same[0]].view(np.uint16), results[other].view(np.uint16)), (same[0], other)
 
 
 @pytest.mark.parametrize("m_batch", [4, 11])

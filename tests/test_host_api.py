@@ -198,12 +198,12 @@ def test_gemv_argument_checks_return_codes_without_launching():
     assert lib.mgemv_dequantize(p, p, p, p, 64, 512, 16, 2, 4, None) == 5
     # per-column mode ignores group_size entirely (mixed_gemv_test.cu:142-143): 16 would be rejected otherwise
     assert lib.mgemv_dequantize(p, p, None, None, 64, 512, 16, 1, 4, None) == 1
-    out = (ctypes.c_int * 7)()
+    out = (ctypes.c_int * 8)()
     assert lib.mgemv_query_launch(4096, 1, 4096, 4, ctypes.byref(out)) == 0
     assert out[0] % 8 == 0 and out[1] % 64 == 0 and out[2] * out[4] >= 8
     assert lib.mgemv_query_launch(4096, 1, 4096, 3, ctypes.byref(out)) == 7
-    assert lib.mgemv_set_launch_override(-1, 0, 0) == 10
-    assert lib.mgemv_set_launch_override(0, 0, 3) == 10
+    assert lib.mgemv_set_launch_override(-1, 0, 0, 0) == 10
+    assert lib.mgemv_set_launch_override(0, 0, 3, 0) == 10
     assert lib.mgemv_set_matrix_core_threshold(18) == 8
 
 
