@@ -34,7 +34,8 @@ __device__ __forceinline__ half2_t splat(half_t v) { return half2_t{v, v}; }
 struct ConvertRegs {
   uint32_t mask7;     // 0x07800780   the 4-bit field at bits 7-10 of each 16-bit half
   uint32_t mask3;     // 0x00780078   the 4-bit field at bits 3-6 of each 16-bit half
-  uint32_t magic;     // 0x64006400   fp16 1024.0 in both halves
+  uint32_t magic;     // 0x64006400   fp16 1024.0 in both halves      (general form only)
+  uint32_t minus136;  // 0xd840d840   fp16 -136.0 in both halves      (general form only)
   uint32_t sel_lo;    // v_perm selector: bytes 0,1 of a word into the low byte of each half
   uint32_t sel_hi;    // v_perm selector: bytes 2,3
 };
@@ -44,13 +45,23 @@ __device__ __forceinline__ ConvertRegs make_convert_regs() {
   c.mask7 = 0x07800780u;
   c.mask3 = 0x00780078u;
   c.magic = 0x64006400u;
+  c.minus136 = 0xd840d840u;
   c.sel_lo = 0x04010400u;
   c.sel_hi = 0x04030402u;
   asm("" : "+s"(c.mask7));
   asm("" : "+s"(c.mask3));
-  asm("" : "+v"(c.magic));
+  asm("" : "+s"(c.magic));     // parked in SGPRs; general_form_regs() moves them where they are needed
+  asm("" : "+s"(c.minus136));
   asm("" : "+s"(c.sel_lo));
   asm("" : "+s"(c.sel_hi));
+  return c;
+}
+
+// The general form needs its two packed constants in VGPRs (a VOP3 instruction reads at most
+// one SGPR).  They are copied there at the start of each general-form unit instead of living
+// in VGPRs for the whole kernel, where they would cost the short form a wave of occupancy.
+__device__ __forceinline__ ConvertRegs general_form_regs(ConvertRegs c) {
+  asm volatile("v_mov_b32 %0, %2\n\tv_mov_b32 %1, %3" : "=&v"(c.magic), "=v"(c.minus136) : "s"(c.magic), "s"(c.minus136));
   return c;
 }
 
@@ -70,7 +81,7 @@ __device__ __forceinline__ void convert_int4_word(uint32_t w, const ConvertRegs&
   const half2_t h2 = as_half2((__builtin_amdgcn_alignbit(w, w, 12) & c.mask3) | c.magic);
   const half2_t h3 = as_half2(((w >> 8) & c.mask3) | c.magic);
   const half2_t k8th = splat((half_t)0.125f);
-  const half2_t kn136 = splat((half_t)-136.0f);
+  const half2_t kn136 = as_half2(c.minus136);
   q[0] = __builtin_elementwise_fma(h0, k8th, kn136);
   q[1] = __builtin_elementwise_fma(h1, k8th, kn136);
   q[2] = __builtin_elementwise_fma(h2, k8th, kn136);
