@@ -49,7 +49,7 @@ WORKLOADS = {
 # averaged over the launches of `bench.py --workload <name> --launch stream`), scaled by what the same
 # counters read for a plain 512 MiB device copy on the same box: FETCH_SIZE reads 262155.5 for 524288 KiB
 # (factor 2.0), WRITE_SIZE reads 524288 (factor 1.0).  See profiles/.  name -> (fetch KiB raw, write KiB raw)
-MEASURED_TRAFFIC_KIB = {"ns": (4460.5, 8.0), "c5": (61068.5, 56.0)}
+MEASURED_TRAFFIC_KIB = {"ns": (4471.5, 8.0), "c5": (61086.0, 56.0)}
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
 
@@ -260,6 +260,9 @@ def main():
                          "rotation of the buffer sets per replay); stream: one host launch per step")
     ap.add_argument("--extra", default="c5", help="comma list of further workloads reported under 'other_workloads' ('' = none)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / oracle check")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only copy 512 MiB device to device four times and exit: the known-size kernel against which "
+                         "the FETCH_SIZE / WRITE_SIZE counters of `rocprofv3 --pmc` are scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (a GEMV over one weight matrix held by one MI355X); "
@@ -273,6 +276,16 @@ def main():
     import mixed_gemv_amd as mg
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.copy_calibration:
+        n = 512 << 20
+        src = torch.full((n,), 3, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copied_bytes_per_kernel": n, "kernels": 4}))
+        return
 
     wl = Workload(args.workload, device, m_batch=args.m_batch)
     wall, ev_us, steps, warm_done = time_workload(wl, args.steps, args.warmup, use_graph=(args.launch == "graph"))
