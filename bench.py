@@ -133,9 +133,27 @@ class Workload:
         self.mg = mg
 
     def launch(self, i):
+        if getattr(self, "batch", 0):
+            return self.launch_batched(i)
         j = i % self.sets
         self.mg.device_gemv(self.w[j], self.x, self.s[j], self.z[j], self.bias, self.y, 1, self.n_out, self.m_batch,
                             self.k, self.group, self.quant_op, self.bits)
+
+    def enable_batched(self, batch):
+        """Later launches run `batch` consecutive buffer sets as ONE batched launch (the reference's
+        batch_count / batch strides, gemv/device/gemv_adaptor.h:129-135): independent problems that
+        share the activations."""
+        import torch
+        self.batch = batch
+        self.set_stride = (self.w[1].data_ptr() - self.w[0].data_ptr()) if self.sets > 1 else 0
+        self.y_batched = torch.zeros((batch, self.m_batch, self.n_out), dtype=torch.half, device=self.y.device)
+
+    def launch_batched(self, i):
+        b = self.batch
+        j = (i % (self.sets // b)) * b
+        self.mg.device_gemv(self.w[j], self.x, self.s[j], self.z[j], self.bias, self.y_batched, b, self.n_out,
+                            self.m_batch, self.k, self.group, self.quant_op, self.bits,
+                            batch_strides=(self.set_stride, 0, self.set_stride // 2, 0, self.m_batch * self.n_out))
 
     def host_operands(self, j=0):
         np = self.np
@@ -258,7 +276,9 @@ def main():
     ap.add_argument("--launch", default="graph", choices=["graph", "stream"],
                     help="graph: the steps are replayed from a captured HIP graph (one kernel node per step, one "
                          "rotation of the buffer sets per replay); stream: one host launch per step")
-    ap.add_argument("--extra", default="c5", help="comma list of further workloads reported under 'other_workloads' ('' = none)")
+    ap.add_argument("--extra", default="c5,nsx8,nsx16",
+                    help="comma list of further workloads reported under 'other_workloads' ('' = none); "
+                         "'<name>x<B>' runs B problems per launch through the batched entry point")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / oracle check")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy 512 MiB device to device four times and exit: the known-size kernel against which "
@@ -332,12 +352,20 @@ def main():
                          "ok": bool(chk["max_rel_err"] <= 2e-3)}
     others = {}
     for name in [n for n in args.extra.split(",") if n and n != args.workload]:
-        w2 = Workload(name, device)
-        wall2, ev2, st2, _ = time_workload(w2, max(200, args.steps // 8), max(20, args.warmup // 4), use_graph=(args.launch == "graph"))
-        others[name] = {"workload": w2.description, "us_per_call": round(wall2 * 1e6 / st2, 3),
-                        "value_GBps": round(w2.bytes / (wall2 / st2) / 1e9, 1),
+        # "<workload>x<B>": B problems per launch through the batched entry point
+        base, _, batch = name.partition("x")
+        batch = int(batch) if batch else 1
+        w2 = Workload(base, device, min_sets=5 * batch if batch > 1 else None)
+        if batch > 1:
+            w2.enable_batched(batch)
+        wall2, ev2, st2, _ = time_workload(w2, max(200, args.steps // (8 * batch)), max(20, args.warmup // 4),
+                                           use_graph=(args.launch == "graph"))
+        others[name] = {"workload": w2.description + (f", {batch} independent problems per launch" if batch > 1 else ""),
+                        "us_per_call": round(wall2 * 1e6 / st2, 3),
+                        "us_per_problem": round(wall2 * 1e6 / st2 / batch, 3),
+                        "value_GBps": round(batch * w2.bytes / (wall2 / st2) / 1e9, 1),
                         "kernel_us_avg_events": round(ev2, 3),
-                        "roofline_frac": round(w2.bytes / (ev2 * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                        "roofline_frac": round(batch * w2.bytes / (ev2 * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                         "buffer_sets_rotated": w2.sets, "steps": st2}
         del w2
         torch.cuda.empty_cache()

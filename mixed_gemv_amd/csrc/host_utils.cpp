@@ -247,6 +247,6 @@ const char* mgemv_status_string(int status) {
   }
 }
 
-int mgemv_version(void) { return 100; }
+int mgemv_version(void) { return 200; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
 
 }  // extern "C"
