@@ -300,14 +300,25 @@ def test_batched_launch_with_strides(gpu):
     x = torch.from_numpy(probs[0].x.view(np.int16)).to(gpu)
     y = torch.full((e, n_out), 0x7E00, dtype=torch.int16, device=gpu)
     groups = k // g
-    mg.device_gemv(w, x, scale, zero, bias, y, e, n_out, 1, k, g, SCALE_AND_ZEROS, 4,
-                   batch_strides=(one, 0, groups * n_out, n_out, n_out))
-    torch.cuda.synchronize()
-    got = y.cpu().numpy().view(np.float16)
-    for i, p in enumerate(probs):
-        p.x = probs[0].x
-        _, rel, _ = error_report(got[i], p.oracle_gemv(threads=8)[0])
-        assert rel <= REL_TOL, i
+    results = []
+    try:
+        # default geometry, then one workgroup per problem (every wave walks all four tiles in a row)
+        for cap in (0, 1):
+            mg.set_launch_override(0, 0, 0, cap)
+            y.fill_(0x7E00)
+            mg.device_gemv(w, x, scale, zero, bias, y, e, n_out, 1, k, g, SCALE_AND_ZEROS, 4,
+                           batch_strides=(one, 0, groups * n_out, n_out, n_out))
+            torch.cuda.synchronize()
+            results.append(y.cpu().numpy().view(np.float16).copy())
+    finally:
+        mg.set_launch_override(0, 0, 0, 0)
+    assert mg.query_launch(n_out, 1, k, 4)["tiles_in_sequence"] == 1
+    for got in results:
+        for i, p in enumerate(probs):
+            p.x = probs[0].x
+            _, rel, _ = error_report(got[i], p.oracle_gemv(threads=8)[0])
+            assert rel <= REL_TOL, i
+    assert np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))   # same k split, same sums
 
 
 def test_adaptor_mirror_runs(gpu):
