@@ -240,6 +240,32 @@ def time_workload(wl, steps, warmup, use_graph=False):
     return wall, e0.elapsed_time(e1) * 1e3 / steps, steps, done
 
 
+def launch_floor_us(device):
+    """Cadence of the smallest possible kernel (a one-element fill) replayed from a HIP graph like the
+    timed steps: what one launch costs on this machine before it reads a single byte."""
+    import torch
+    cell = torch.zeros(1, dtype=torch.int32, device=device)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(64):
+                cell.fill_(1)
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(20):
+        graph.replay()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(100):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / 6400
+
+
 def check_against_oracle(wl, rows=None):
     """GPU result of buffer set 0 against the CPU oracle on the first `rows` rows; also times
     the oracle single-threaded (the reference's HOST_CHECK loop has no threading)."""
@@ -375,6 +401,11 @@ def main():
     wl.sets = all_sets
     out["warm_cache"] = {"us_per_call": round(wall_w * 1e6 / st_w, 3), "GBps": round(wl.bytes / (wall_w / st_w) / 1e9, 1),
                          "note": "one buffer set re-read from the 256 MB Infinity Cache; not an HBM figure"}
+    if args.launch == "graph":
+        floor = launch_floor_us(device)
+        out["launch_floor"] = {"us_per_launch": round(floor, 3),
+                               "kernel_us_above_floor": round(kernel_us - floor, 3),
+                               "note": "graph replay of a one-element fill kernel: the cadence of an empty launch"}
     if not args.no_cpu:
         chk = check_against_oracle(wl)
         out["cpu_baseline"] = {
