@@ -106,8 +106,9 @@ MGEMV_API size_t mgemv_preprocessed_size(const size_t *shape, int rank, int quan
  *   quant_type MGEMV_W4_A16 or MGEMV_W8_A16 (the reference's interleave rejects W8_A16,
  *           utils/preprocess.h:350-362; here both are laid out).
  * Same input meaning as the reference, different OUTPUT layout: the gfx950 tile layout
- * consumed by mgemv_gemv (16-row tiles, 1 KiB wave-contiguous blocks, biased nibbles in
- * converter order).  dst must hold mgemv_preprocessed_size() bytes and may not alias src. */
+ * consumed by mgemv_gemv (16-row tiles, 1 KiB wave-contiguous blocks, biased 4-bit fields at
+ * the bit positions the dequantiser masks out directly).  The layout belongs to this library
+ * version (mgemv_version).  dst must hold mgemv_preprocessed_size() bytes and may not alias src. */
 MGEMV_API int mgemv_preprocess_weights(uint8_t *dst, const uint8_t *src, const size_t *shape, int rank,
                                        int layout, int quant_type);
 

@@ -1,12 +1,13 @@
 // GEMV and dequantise kernels for gfx950 (MI355X), wave64, plus their C-ABI launchers.
 //
-// One wavefront works on one 16-row tile of the weight matrix and a contiguous range of k
-// steps (units of tile_layout.h).  Per unit it issues four 1-KiB weight loads, one activation
-// load and the scale/zero loads, converts and dequantises in packed fp16 (two roundings, as
-// gemv/warp/warp_dequantizer.h:52-59), and accumulates in fp32 with v_dot2c_f32_f16 whose
-// activation operand is a DPP row broadcast.  Several waves of a workgroup split the k range
-// of the same tile (split-K); their per-lane partial sums meet in LDS, are summed in a fixed
-// order, biased, rounded to fp16 and stored.  This covers, for the reference, the main loops
+// One wavefront works on a contiguous range of k steps (units of tile_layout.h) of one 16-row
+// tile of the weight matrix, or of several consecutive tiles one after the other.  Per unit it
+// issues four 1-KiB weight loads, one activation load and the scale/zero loads, dequantises
+// in packed fp16 to the bits of gemv/warp/warp_dequantizer.h:52-59 (rounded product, then
+// rounded sum), and accumulates in fp32 with v_dot2c_f32_f16 whose activation operand is a DPP
+// row broadcast.  Several waves of a workgroup split the k range of the same tiles (split-K);
+// their per-lane partial sums meet in LDS, are summed in a fixed order, biased, rounded to
+// fp16 and stored.  This covers, for the reference, the main loops
 // of gemv/threadblock/dq_mma_singlestage_{finegrained,percol}.h, the reductions of
 // gemv/warp/reduce.h and gemv/threadblock/accumulator_combine.h, and the epilogue of
 // epilogue/threadblock/epilogue.h.
@@ -653,8 +654,7 @@ __device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<
 
 // blockDim = (64 * split_k, tiles_per_wg); each wave works on T consecutive tiles so that the
 // activation operands of a k step are fetched once and used T times.  Dynamic LDS:
-// tiles_per_wg * split_k * T * 256 floats (none when split_k == 1).  m_batch travels in
-// tail.reserved.
+// tiles_per_wg * split_k * T * 256 floats (none when split_k == 1).
 template <int BITS, int QOP, int GROUPS_PER_RUN, int T>
 __global__ void __launch_bounds__(kWave * kMaxWavesPerMfmaWorkgroup)
 gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
