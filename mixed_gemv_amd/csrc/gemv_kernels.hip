@@ -453,9 +453,9 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
 
     // Two fragments in flight: the loads of unit u+1 are issued before unit u is computed, so
     // a wave that is waiting for its turn on the VALU still has memory requests outstanding.
-    // The first unit is requested on its own, ahead of the loop: when a whole launch is only
-    // two units per wave, asking for everything at once would only put every wave's first unit
-    // behind everybody's second one in the memory queues.
+    // (The first fragment is loaded ahead of the loop and reaches it through register copies,
+    // which wait for its data before the second unit is requested.  A loop that loads both
+    // fragments inside, without that wait, measured the same to 2 % on every shape.)
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
     load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
     const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
