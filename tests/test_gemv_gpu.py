@@ -240,6 +240,40 @@ def test_split_k_invariance_and_determinism(gpu):
             assert np.array_equal(results[same[0]].view(np.uint16), results[other].view(np.uint16)), (same[0], other)
 
 
+WALKS = [
+    # tag, n_out, k, bits, quant_op, group, m_batch, bias
+    ("w_i4_sz_g64", 208, 2048, 4, SCALE_AND_ZEROS, 64, 1, True),     # two groups per lane run
+    ("w_i4_sz_g160", 100, 1120, 4, SCALE_AND_ZEROS, 160, 1, True),   # generic group lookup, ragged rows and k
+    ("w_i4_col", 176, 1536, 4, PER_COLUMN, 0, 2, False),
+    ("w_i4_s_g128_mb3", 144, 1024, 4, SCALE_ONLY, 128, 3, True),
+    ("w_i8_sz_g128", 112, 768, 8, SCALE_AND_ZEROS, 128, 1, False),
+    ("w_i8_col_mb4", 96, 512, 8, PER_COLUMN, 0, 4, True),
+]
+
+
+@pytest.mark.parametrize("cfg", WALKS, ids=[c[0] for c in WALKS])
+def test_tile_walks_match_one_tile_per_wave(gpu, cfg):
+    """Every kernel variant with waves that walk several tiles in a row (fewer workgroups than
+    tiles): same bits as the one-tile-per-wave launch with the same k split, and parity with the oracle."""
+    tag, n_out, k, bits, qop, g, mb, bias = cfg
+    prob = Problem(tag, n_out, k, bits, qop, g, m_batch=mb, bias=bias)
+    dev = DeviceProblem(prob, gpu)
+    ref = prob.oracle_gemv(threads=16)
+    try:
+        for sk in (1, 2):
+            mg.set_launch_override(sk, 1, 0, 0)
+            base = dev.run().copy()
+            _, rel, _ = error_report(base, ref)
+            assert rel <= REL_TOL, (sk, rel)
+            for tw, cap in ((1, 3), (2, 2), (1, 1)):
+                mg.set_launch_override(sk, tw, 0, cap)
+                assert mg.query_launch(n_out, mb, k, bits)["tiles_in_sequence"] > 1
+                got = dev.run().copy()
+                assert np.array_equal(got.view(np.uint16), base.view(np.uint16)), (sk, tw, cap)
+    finally:
+        mg.set_launch_override(0, 0, 0, 0)
+
+
 @pytest.mark.parametrize("m_batch", [4, 11])
 def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     """Rows of a batch are independent GEMVs.  Up to 4 rows the VALU kernel adds every row in
