@@ -383,6 +383,25 @@ FULL = [
 ]
 
 
+# Shapes that take the other branches of the launch heuristic (one four-wave workgroup per compute
+# unit with 4 / 2 / 1 tile sequences, with and without several tiles per sequence, with remainders).
+FIT = [
+    ("fit_tw4_two_tiles_each", 32032, 2048, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
+    ("fit_tw2_long_k", 8192, 28672, 4, SCALE_AND_ZEROS, 128, 1, True, "normal", (0.001, 0.02)),
+    ("fit_vocab", 128256, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
+    ("fit_int8_tw2", 8192, 4096, 8, PER_COLUMN, 0, 2, True, "uniform", (0.001, 0.01)),
+]
+
+
+@pytest.mark.parametrize("cfg", FIT, ids=[c[0] for c in FIT])
+def test_exact_fit_launches_full_size(gpu, cfg):
+    tag, n_out, k, bits, qop, g, mb, bias, xd, sr = cfg
+    plan = mg.query_launch(n_out, mb, k, bits)
+    assert plan["workgroups"] == 256 and plan["threads"] == 256, plan
+    prob = Problem(tag, n_out, k, bits, qop, g, m_batch=mb, bias=bias, x_dist=xd, scale_range=sr)
+    check(prob, gpu, dequant=False)
+
+
 @pytest.mark.parametrize("cfg", FULL, ids=[c[0] for c in FULL])
 def test_baseline_configs_full_size(gpu, cfg):
     tag, n_out, k, bits, qop, g, mb, bias, xd, sr = cfg
