@@ -14,9 +14,12 @@ SOURCES = ["gemv_kernels.hip", "host_utils.cpp"]
 
 # -ffp-contract=off: the dequantiser is a separately rounded fp16 multiply and add.
 # -packed-fp32-ops off: keep the compiler from forming v_pk_*_f32.
+# -amdgpu-kernarg-preload-count=14: the first 14 dwords of kernel arguments arrive in SGPRs with
+# the wave (measured: 0.1 us off the 4 us launches).
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-fvisibility=hidden", "-DMGEMV_BUILDING_LIBRARY", "-fopenmp",
     "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]

@@ -30,9 +30,9 @@ constexpr int kNumCus = 256;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
 
-// Kernel arguments.  The first ten (four pointers and six 32-bit words) are what a wave needs
-// to address its first loads; everything else sits in GemvTail.  The kernels pull ALL of
-// them into SGPRs with one batch of scalar loads at entry (see the asm statement there).
+// Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are what a
+// wave needs to address its first loads, and they are preloaded into SGPRs (build flag
+// -amdgpu-kernarg-preload-count=14); everything else sits in GemvTail.
 struct GemvTail {
   const half_t* bias;
   half_t* y;
@@ -376,7 +376,7 @@ template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI>
 __global__ void __launch_bounds__(kWave * (MB >= 3 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
 __attribute__((amdgpu_waves_per_eu(MB == 1 && GROUPS_PER_RUN == 1 ? 6 : 1)))
 gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
-                uint32_t packed_steps, int workgroups, int wgs_per_xcd, uint32_t packed_group, GemvTail tail) {
+                uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
   extern __shared__ float partials[];
   Problem p;
   p.weights = weights;
@@ -388,22 +388,22 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   p.ksteps = (int)(packed_steps & 0xffffu);
   p.steps_per_wave = (int)(packed_steps >> 16);
   p.workgroups = workgroups;
-  p.wgs_per_xcd = wgs_per_xcd;
+  p.wgs_per_xcd = (workgroups + kNumXcd - 1) / kNumXcd;
   p.group_size = (int)(packed_group & 0xffffffu);
   p.tiles_per_wg = (int)(packed_group >> 24);
-  // Bring every kernel argument into SGPRs with ONE round trip to memory.  Left alone, the
-  // compiler sinks each scalar load next to its first use, which puts three or four dependent
-  // load-wait pairs in front of the first weight load of these microsecond-scale kernels.
-  asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
-               "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
-               "s"(tail.num_groups), "s"(tail.flags), "s"(tail.seq_base), "s"(tail.seq_rem), "s"(tail.stride_weights),
-               "s"(tail.stride_x), "s"(tail.stride_scale), "s"(tail.stride_bias), "s"(tail.stride_y));
-  // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223); branch-free.
+  // The library is built with kernel-argument preloading: the four pointers and six words in
+  // front of GemvTail arrive in SGPRs with the wave (firmware without the feature runs a short
+  // prologue that loads them instead).  Nothing on the way to the first weight loads of an
+  // unbatched launch reads the tail, so those loads do not wait for any scalar load at all.
+  // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223): problems past the first fetch
+  // their strides first.
   const long long batch = blockIdx.z;
-  p.weights += batch * tail.stride_weights;
-  p.x += batch * tail.stride_x;
-  p.scale += batch * tail.stride_scale;
-  p.zero_add += batch * tail.stride_scale;  // only dereferenced in scale+zero mode
+  if (batch != 0) {
+    p.weights += batch * tail.stride_weights;
+    p.x += batch * tail.stride_x;
+    p.scale += batch * tail.stride_scale;
+    p.zero_add += batch * tail.stride_scale;  // only dereferenced in scale+zero mode
+  }
   const bool has_bias = tail.bias != nullptr;
   tail.bias += batch * tail.stride_bias;
   tail.y += batch * tail.stride_y;
@@ -438,7 +438,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
 #pragma unroll
     for (int m = 0; m < MB; ++m) x_rsrc[m] = make_rsrc(p.x + (size_t)m * (size_t)p.k, (uint32_t)p.k * 2u);
     ScaleTables tables;
-    const uint32_t table_bytes = (uint32_t)tail.num_groups * (uint32_t)p.n_out * 2u;
+    const uint32_t table_bytes = (uint32_t)num_groups * (uint32_t)p.n_out * 2u;
     tables.scale = make_rsrc(p.scale, table_bytes);
     tables.zero = make_rsrc(p.zero_add, QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? table_bytes : 0u);
     TileWalk walk;
@@ -1032,7 +1032,7 @@ template <int BITS, int QOP, int MB, int GPR, bool MULTI>
 hipError_t launch_gemv_kernel_m(const GemvLaunch& g) {
   return launch(gemv_dpp_kernel<BITS, QOP, MB, GPR, MULTI>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
                 g.zero_add, g.n_out, g.k, pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups,
-                g.plan.wgs_per_xcd, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+                g.tail.num_groups, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
 }
 
 template <int BITS, int QOP, int MB, int GPR>
