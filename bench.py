@@ -49,7 +49,7 @@ WORKLOADS = {
 # averaged over the launches of `bench.py --workload <name> --launch stream`), scaled by what the same
 # counters read for a plain 512 MiB device copy on the same box: FETCH_SIZE reads 262155.5 for 524288 KiB
 # (factor 2.0), WRITE_SIZE reads 524288 (factor 1.0).  See profiles/.  name -> (fetch KiB raw, write KiB raw)
-MEASURED_TRAFFIC_KIB = {"ns": (4471.5, 8.0), "c5": (61086.0, 56.0)}
+MEASURED_TRAFFIC_KIB = {"ns": (4472.0, 8.0), "c5": (61082.5, 56.0)}
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
 
@@ -335,6 +335,8 @@ def main():
                     help="comma list of further workloads reported under 'other_workloads' ('' = none); "
                          "'<name>x<B>' runs B problems per launch through the batched entry point")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / oracle check")
+    ap.add_argument("--no-warm-cache", action="store_true",
+                    help="skip the warm-cache and launch-floor side measurements (keeps a kernel trace to the cold launches)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy 512 MiB device to device four times and exit: the known-size kernel against which "
                          "the FETCH_SIZE / WRITE_SIZE counters of `rocprofv3 --pmc` are scaled")
@@ -396,12 +398,14 @@ def main():
     }
     # the same launches on ONE buffer set, i.e. out of the Infinity Cache: reported beside the cold
     # figure, never as `value`
-    all_sets, wl.sets = wl.sets, 1
-    wall_w, ev_w, st_w, _ = time_workload(wl, max(200, args.steps // 4), 20, use_graph=(args.launch == "graph"))
-    wl.sets = all_sets
-    out["warm_cache"] = {"us_per_call": round(wall_w * 1e6 / st_w, 3), "GBps": round(wl.bytes / (wall_w / st_w) / 1e9, 1),
-                         "note": "one buffer set re-read from the 256 MB Infinity Cache; not an HBM figure"}
-    if args.launch == "graph":
+    if not args.no_warm_cache:
+        all_sets, wl.sets = wl.sets, 1
+        wall_w, ev_w, st_w, _ = time_workload(wl, max(200, args.steps // 4), 20, use_graph=(args.launch == "graph"))
+        wl.sets = all_sets
+        out["warm_cache"] = {"us_per_call": round(wall_w * 1e6 / st_w, 3),
+                             "GBps": round(wl.bytes / (wall_w / st_w) / 1e9, 1),
+                             "note": "one buffer set re-read from the 256 MB Infinity Cache; not an HBM figure"}
+    if args.launch == "graph" and not args.no_warm_cache:
         floor = launch_floor_us(device)
         out["launch_floor"] = {"us_per_launch": round(floor, 3),
                                "kernel_us_above_floor": round(kernel_us - floor, 3),
