@@ -177,6 +177,17 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
  * tests.  Process-wide. */
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
+/* Which of the two matrix-core kernels serves the small batches:
+ *   MGEMV_MATRIX_CORE_AUTO (default)          the LDS-staged kernel wherever the matrix has at least two
+ *                                             16-row tiles, else the register-operand kernel;
+ *   MGEMV_MATRIX_CORE_REGISTER_OPERAND        always the kernel that reads its activation operand from
+ *                                             L2 into registers;
+ *   MGEMV_MATRIX_CORE_LDS_STAGED              same choice as AUTO (named for symmetry in tests).
+ * Same results to tolerance either way (the k split, hence the order of the fp32 sums, differs).
+ * For tests and measurements; no counterpart in the reference.  Process-wide. */
+enum { MGEMV_MATRIX_CORE_AUTO = 0, MGEMV_MATRIX_CORE_REGISTER_OPERAND = 1, MGEMV_MATRIX_CORE_LDS_STAGED = 2 };
+MGEMV_API int mgemv_set_matrix_core_variant(int variant);
+
 /* Which int4 dequantiser the kernels may use.  Both produce the same bits, rn16(rn16(q*s) + z)
  * as gemv/warp/warp_dequantizer.h:52-59:
  *   MGEMV_DEQUANT_AUTO (default)    per wave and k step, the one-FMA form wherever every scale
@@ -190,7 +201,8 @@ MGEMV_API int mgemv_set_dequant_form(int form);
 
 /* Reports the geometry mgemv_gemv would use: out[0] = workgroups, out[1] = threads per
  * workgroup, out[2] = k-split waves per tile, out[3] = tile sequences per workgroup,
- * out[4] = k steps per wave and tile, out[5] = 1 when the matrix-core path is chosen,
+ * out[4] = k steps per wave and tile, out[5] = 0 VALU kernel / 1 matrix-core kernel with the
+ * activation operand in registers / 2 LDS-staged matrix-core kernel,
  * out[6] = tiles per wave (matrix-core path), out[7] = most tiles a wave walks one after the
  * other (VALU path). */
 MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8]);

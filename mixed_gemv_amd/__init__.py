@@ -19,6 +19,10 @@ from .api import (  # noqa: F401
     set_launch_override,
     set_matrix_core_threshold,
     set_dequant_form,
+    set_matrix_core_variant,
+    MATRIX_CORE_AUTO,
+    MATRIX_CORE_REGISTER_OPERAND,
+    MATRIX_CORE_LDS_STAGED,
     DEQUANT_AUTO,
     DEQUANT_EXACT_INTEGER,
     unpreprocess_weights,

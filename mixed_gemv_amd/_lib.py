@@ -31,6 +31,7 @@ SIGNATURES = {
     "mgemv_set_launch_override": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int, _c.c_int]),
     "mgemv_set_matrix_core_threshold": (_c.c_int, [_c.c_int]),
     "mgemv_set_dequant_form": (_c.c_int, [_c.c_int]),
+    "mgemv_set_matrix_core_variant": (_c.c_int, [_c.c_int]),
     "mgemv_query_launch": (_c.c_int, [_c.c_int] * 4 + [_c.POINTER(_c.c_int * 8)]),
 }
 

@@ -216,6 +216,16 @@ def set_matrix_core_threshold(min_m_batch=0):
     _lib.check(_lib.lib().mgemv_set_matrix_core_threshold(int(min_m_batch)), "set_matrix_core_threshold")
 
 
+MATRIX_CORE_AUTO = 0
+MATRIX_CORE_REGISTER_OPERAND = 1
+MATRIX_CORE_LDS_STAGED = 2
+
+
+def set_matrix_core_variant(variant=MATRIX_CORE_AUTO):
+    """Which matrix-core kernel serves the small batches; see mgemv_set_matrix_core_variant."""
+    _lib.check(_lib.lib().mgemv_set_matrix_core_variant(int(variant)), "set_matrix_core_variant")
+
+
 DEQUANT_AUTO = 0
 DEQUANT_EXACT_INTEGER = 1
 

@@ -588,9 +588,24 @@ __device__ __forceinline__ void load_weights_mfma(MfmaWeights<BITS, GROUPS_PER_R
   }
 }
 
-template <int BITS, int QOP, int GROUPS_PER_RUN, bool SHORT>
+// Where the activation operand of matrix instruction (block i, fragment j) comes from:
+// registers filled by load_activations_mfma, or the workgroup's LDS stage of the current k step.
+template <int BITS>
+__device__ __forceinline__ u32x4 mfma_operand(const MfmaActivations<BITS>& xa, int i, int j) { return xa.x[i][j]; }
+
+template <int BITS>
+struct LdsActivations {
+  const uint8_t* lane_base;  // row (lane % 16) of the stage, at this lane's k slice
+};
+template <int BITS>
+__device__ __forceinline__ u32x4 mfma_operand(const LdsActivations<BITS>& xa, int i, int j) {
+  using G = Geometry<BITS>;
+  return *reinterpret_cast<const u32x4*>(xa.lane_base + (i * G::kChunkK + j * 8) * 2);
+}
+
+template <int BITS, int QOP, int GROUPS_PER_RUN, bool SHORT, typename Activations>
 __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
-                                                       const MfmaActivations<BITS>& xa, const ConvertRegs& c,
+                                                       const Activations& xa, const ConvertRegs& c,
                                                        half2_t col_scale2) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
 #pragma unroll
@@ -616,8 +631,8 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
         u32x4 a;
 #pragma unroll
         for (int h = 0; h < 4; ++h) a[h] = as_u32(d[h]);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, xa.x[i][j]),
-                                                     acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                     __builtin_bit_cast(half8_t, mfma_operand<BITS>(xa, i, j)), acc, 0, 0, 0);
       }
     } else {
 #pragma unroll
@@ -630,16 +645,16 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
         a[1] = as_u32(dequant_pair<kHasZero>(q0[1], s2, z2));
         a[2] = as_u32(dequant_pair<kHasZero>(q1[0], s2, z2));
         a[3] = as_u32(dequant_pair<kHasZero>(q1[1], s2, z2));
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, xa.x[i][j]),
-                                                     acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
+                                                     __builtin_bit_cast(half8_t, mfma_operand<BITS>(xa, i, j)), acc, 0, 0, 0);
       }
     }
   }
 }
 
-template <int BITS, int QOP, int GROUPS_PER_RUN>
+template <int BITS, int QOP, int GROUPS_PER_RUN, typename Activations>
 __device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
-                                                  const MfmaActivations<BITS>& xa, const ConvertRegs& c,
+                                                  const Activations& xa, const ConvertRegs& c,
                                                   half2_t col_scale2, bool short_allowed) {
   if constexpr (BITS == 4) {
     bool take_short = short_allowed;
@@ -790,6 +805,228 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   }
 }
 
+// Weights, scales and zeros of unit `unit` of the wave's k range through descriptors: everything
+// unit-dependent sits in the bounds-checked VGPR offset, so a prefetch past the range reads zeros.
+template <int BITS, int QOP, int GROUPS_PER_RUN>
+__device__ __forceinline__ void load_weights_lds_mfma(MfmaWeights<BITS, GROUPS_PER_RUN>& f, const Problem& p,
+                                                      __amdgpu_buffer_rsrc_t w_rsrc, const ScaleTables& tables, int unit,
+                                                      int kstep, int lane, int row) {
+  using G = Geometry<BITS>;
+  const int voffset = unit * kUnitBytes + lane * kChunkBytes;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i)
+    f.w[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, voffset + i * kBlockBytes, 0, kCacheStream);
+  if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) {
+    const int k_run = kstep * G::kStepK + (lane / kTileRows) * G::kRunK;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) {
+      const int grp = group_of(p, k_run + gi * (G::kRunK / GROUPS_PER_RUN));
+      const int off = (grp * p.n_out + row) * 2;
+      f.s[gi] = load_b16_low(tables.scale, off);
+      if constexpr (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS) f.z[gi] = load_b16_low(tables.zero, off);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Small-batch variant on the matrix cores with the activation operand staged through LDS.
+//
+// The kernel above reads its activation operand -- 16 rows x 512 k = 16 KiB per k step -- from
+// L2 into registers, sixteen 128-bit loads per lane and step; that leaves no registers for
+// prefetching, so it hides latency by occupancy alone.  Here the tiles_per_wg waves of a
+// workgroup that work on the SAME k range (different tiles) fetch that slice once, together,
+// into a double-buffered LDS stage: round r of wave ty brings one whole row (64 lanes x 16
+// bytes) of batch row ty + r * tiles_per_wg.  The matrix instructions read their operand from
+// LDS just in time (rows 1040 bytes apart, so the 16 lanes of a k slice hit 16 distinct bank
+// groups), the registers hold two k steps of weights, and the global loads of step u+1 -- weights
+// and activation rows -- are in flight while step u is computed.  One barrier per k step.
+// ROUNDS = staged rows / tiles_per_wg; staged rows (8 or 16) >= m_batch.  Lanes of batch rows
+// that are not staged read some other row: columns of a matrix product do not mix, and those
+// columns are never stored.
+// ---------------------------------------------------------------------------------------------
+template <int BITS>
+struct XStage {
+  static constexpr int kRowBytes = Geometry<BITS>::kStepK * 2;  // 1024 | 512
+  static constexpr int kRowStride = kRowBytes + 16;             // bank spread for the operand reads
+  static constexpr int kLaneBytes = kRowBytes / kWave;          // 16 | 8
+};
+
+template <int BITS, int ROUNDS>
+struct XRows {
+  uint32_t v[ROUNDS][BITS == 4 ? 4 : 2];
+};
+
+template <int BITS, int ROUNDS>
+__device__ __forceinline__ void fetch_x_rows(XRows<BITS, ROUNDS>& r, const Problem& p, __amdgpu_buffer_rsrc_t x_rsrc,
+                                             int kstep, int lane, int first_row, int row_step) {
+  using G = Geometry<BITS>;
+  const int k0 = kstep * G::kStepK + lane * (XStage<BITS>::kLaneBytes / 2);
+#pragma unroll
+  for (int j = 0; j < ROUNDS; ++j) {
+    const int row = first_row + j * row_step;
+    // rows past m_batch fall outside the descriptor, reduction positions past k are sent there
+    const uint32_t off = k0 < p.k ? (uint32_t)(row * p.k + k0) * 2u : 0xfffffff0u;
+    if constexpr (BITS == 4) {
+      const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, kCacheDefault);
+      r.v[j][0] = t[0]; r.v[j][1] = t[1]; r.v[j][2] = t[2]; r.v[j][3] = t[3];
+    } else {
+      const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(x_rsrc, (int)off, 0, kCacheDefault);
+      r.v[j][0] = t[0]; r.v[j][1] = t[1];
+    }
+  }
+}
+
+template <int BITS, int ROUNDS>
+__device__ __forceinline__ void park_x_rows(const XRows<BITS, ROUNDS>& r, uint8_t* stage, int lane, int first_row,
+                                            int row_step) {
+#pragma unroll
+  for (int j = 0; j < ROUNDS; ++j) {
+    uint8_t* dst = stage + (first_row + j * row_step) * XStage<BITS>::kRowStride + lane * XStage<BITS>::kLaneBytes;
+    if constexpr (BITS == 4) {
+      *reinterpret_cast<u32x4*>(dst) = u32x4{r.v[j][0], r.v[j][1], r.v[j][2], r.v[j][3]};
+    } else {
+      *reinterpret_cast<u32x2*>(dst) = u32x2{r.v[j][0], r.v[j][1]};
+    }
+  }
+}
+
+// blockDim = (64 * split_k, tiles_per_wg), at most 8 waves.  Dynamic LDS: split_k * 2 stages of
+// (ROUNDS * tiles_per_wg) rows x kRowStride bytes, then tiles_per_wg * split_k * 256 floats for
+// the split-K combine.
+template <int BITS, int QOP, int GROUPS_PER_RUN, int ROUNDS>
+__global__ void __launch_bounds__(kWave * kMaxWavesPerMfmaWorkgroup)
+gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out,
+                     int k, uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
+  extern __shared__ float partials[];
+  using XS = XStage<BITS>;
+  Problem p;
+  p.weights = weights;
+  p.x = x;
+  p.scale = scale;
+  p.zero_add = zero_add;
+  p.n_out = n_out;
+  p.k = k;
+  p.ksteps = (int)(packed_steps & 0xffffu);
+  p.steps_per_wave = (int)(packed_steps >> 16);
+  p.workgroups = workgroups;
+  p.wgs_per_xcd = (workgroups + kNumXcd - 1) / kNumXcd;
+  p.group_size = (int)(packed_group & 0xffffffu);
+  p.tiles_per_wg = (int)(packed_group >> 24);
+  const long long batch = blockIdx.z;
+  if (batch != 0) {
+    p.weights += batch * tail.stride_weights;
+    p.x += batch * tail.stride_x;
+    p.scale += batch * tail.stride_scale;
+    p.zero_add += batch * tail.stride_scale;
+  }
+  const bool has_bias = tail.bias != nullptr;
+  tail.bias += batch * tail.stride_bias;
+  tail.y += batch * tail.stride_y;
+  const int m_batch = tail.m_batch;
+
+  const int wg = logical_workgroup(p);
+  if (wg >= p.workgroups) return;  // whole workgroup leaves before any barrier
+
+  const int lane = threadIdx.x % kWave;
+  const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);
+  const int split_k = tail.split_k;
+  const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
+  const int tile_raw = wg * p.tiles_per_wg + ty;
+  const int tile = tile_raw < tiles ? tile_raw : tiles - 1;  // a wave without a tile still stages rows and meets the barriers
+  const int row_raw = tile * kTileRows + lane % kTileRows;
+  const int row = row_raw < p.n_out ? row_raw : p.n_out - 1;
+
+  const int staged_rows = ROUNDS * p.tiles_per_wg;
+  const int stage_bytes = staged_rows * XS::kRowStride;
+  uint8_t* const lds = reinterpret_cast<uint8_t*>(partials);
+  uint8_t* const my_stages = lds + kw * 2 * stage_bytes;  // the two stages of this k range
+  // this lane's operand row: batch row lane % 16 if staged, else any staged row (never stored)
+  const int m_read = (lane % kTileRows) & (staged_rows - 1);
+  const int operand_offset = m_read * XS::kRowStride + (lane / kTileRows) * Geometry<BITS>::kRunK * 2;
+
+  const int steps = p.steps_per_wave;  // the same for every wave: the barriers are workgroup-wide
+  const int ks_begin = kw * steps;
+  const int units = min(ks_begin + steps, p.ksteps) - ks_begin;  // >= 1 by the host's geometry
+  const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
+      p.weights + ((size_t)tile * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
+      (uint32_t)units * (uint32_t)kUnitBytes);
+  const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(p.x, (uint32_t)m_batch * (uint32_t)p.k * 2u);
+  ScaleTables tables;
+  const uint32_t table_bytes = (uint32_t)num_groups * (uint32_t)p.n_out * 2u;
+  tables.scale = make_rsrc(p.scale, table_bytes);
+  tables.zero = make_rsrc(p.zero_add, QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? table_bytes : 0u);
+
+  half2_t col_scale = half2_t{};
+  bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
+  if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+    col_scale = splat(p.scale[row]);
+    const uint32_t bits[1] = {as_u32(col_scale)};
+    short_ok = short_ok && wave_scales_permit_short_form(bits);
+  }
+  const ConvertRegs c = make_convert_regs();
+
+  f32x4 acc = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  XRows<BITS, ROUNDS> xr;
+  MfmaWeights<BITS, GROUPS_PER_RUN> wa, wb;
+  fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin, lane, ty, p.tiles_per_wg);
+  load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wa, p, w_rsrc, tables, 0, ks_begin, lane, row);
+  int u = 0;
+  do {
+    // even step: weights in wa, stage 0
+    park_x_rows<BITS, ROUNDS>(xr, my_stages, lane, ty, p.tiles_per_wg);
+    __syncthreads();
+    fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin + u + 1, lane, ty, p.tiles_per_wg);
+    load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wb, p, w_rsrc, tables, u + 1, ks_begin + u + 1, lane, row);
+    __builtin_amdgcn_sched_barrier(0);
+    if (u < units) {
+      const LdsActivations<BITS> xa{my_stages + operand_offset};
+      compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc, wa, xa, c, col_scale, short_ok);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (u + 1 < steps) {
+      // odd step: weights in wb, stage 1
+      park_x_rows<BITS, ROUNDS>(xr, my_stages + stage_bytes, lane, ty, p.tiles_per_wg);
+      __syncthreads();
+      fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin + u + 2, lane, ty, p.tiles_per_wg);
+      load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wa, p, w_rsrc, tables, u + 2, ks_begin + u + 2, lane, row);
+      __builtin_amdgcn_sched_barrier(0);
+      if (u + 1 < units) {
+        const LdsActivations<BITS> xa{my_stages + stage_bytes + operand_offset};
+        compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc, wb, xa, c, col_scale, short_ok);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    u += 2;
+  } while (u < steps);
+
+  // Lane l holds D[rows 4*(l/16) .. +3 of the tile][batch row l % 16].
+  f32x4 sum = acc;
+  if (split_k > 1) {
+    f32x4* const combine = reinterpret_cast<f32x4*>(lds + split_k * 2 * stage_bytes);
+    combine[(ty * split_k + kw) * kWave + lane] = acc;
+    __syncthreads();
+    if (kw != 0) return;
+    const f32x4* part = combine + ty * split_k * kWave + lane;
+    sum = part[0];
+    for (int w = 1; w < split_k; ++w) sum += part[w * kWave];
+  }
+  if (tile_raw >= tiles) return;
+  const int m = lane % kTileRows;
+  const int n0 = tile * kTileRows + 4 * (lane / kTileRows);
+  if (m < m_batch) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int n = n0 + v;
+      if (n < p.n_out) {
+        float r = sum[v];
+        if (has_bias) r += (float)tail.bias[n];
+        tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
+      }
+    }
+  }
+}
+
 struct DequantParams {
   const uint8_t* weights;
   const half_t* scale;
@@ -873,6 +1110,7 @@ std::atomic<int> g_override_tiles_per_wave{0};
 std::atomic<int> g_override_workgroups{0};
 std::atomic<int> g_matrix_core_min_batch{5};  // m_batch from which the matrix-core kernel is used
 std::atomic<int> g_dequant_flags{0};          // kExactIntegerFormOnly or 0
+std::atomic<int> g_matrix_core_variant{MGEMV_MATRIX_CORE_AUTO};
 
 inline bool use_matrix_cores(int m_batch) { return m_batch >= g_matrix_core_min_batch.load(); }
 
@@ -880,6 +1118,7 @@ struct LaunchPlan {
   int split_k, tiles_per_wg, steps_per_wave, workgroups, wgs_per_xcd, threads;
   int tiles_per_wave;  // 1 on the VALU path; 1, 2 or 4 on the matrix-core path
   int tiles_in_sequence;  // VALU path: most tiles any wave walks one after the other
+  int staged_rows;        // LDS-staged matrix-core kernel: 8 or 16 activation rows per stage; 0 = other kernels
 };
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -888,6 +1127,25 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
   const int ov_t = g_override_tiles_per_wave.load();
+  if (use_matrix_cores(m_batch) && g_matrix_core_variant.load() != MGEMV_MATRIX_CORE_REGISTER_OPERAND && tiles >= 2) {
+    // LDS-staged kernel: two tiles per workgroup share the activation stage; k split until the
+    // launch has about 1.5 k waves (measured: 8192x8192 best at 4 k-split waves, 28672x8192 at 1).
+    LaunchPlan lp{};
+    lp.tiles_per_wg = 2;
+    lp.staged_rows = m_batch <= 8 ? 8 : 16;
+    lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
+    int split = 1;
+    while (split < 4 && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split < 1536) split *= 2;
+    if (ov_sk > 0) split = ov_sk > 4 ? 4 : ov_sk;
+    if (split > ksteps) split = ksteps;
+    lp.steps_per_wave = ceil_div(ksteps, split);
+    lp.split_k = ceil_div(ksteps, lp.steps_per_wave);
+    lp.wgs_per_xcd = ceil_div(lp.workgroups, kNumXcd);
+    lp.threads = kWave * lp.split_k * lp.tiles_per_wg;
+    lp.tiles_per_wave = 1;
+    lp.tiles_in_sequence = 1;
+    return lp;
+  }
   // Matrix-core path: a wave that works on T tiles fetches the activation operands of a k step
   // once for all of them.  Measured on 8192 x 8192 (512 tiles): T = 2 is 1.5-1.8x faster than
   // T = 1 at 8-16 activation rows; T = 4 leaves too few waves to cover the load latency.
@@ -950,6 +1208,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   lp.steps_per_wave = steps;
   lp.workgroups = ceil_div(groups, tiles_per_wg);
   lp.tiles_in_sequence = 1;
+  lp.staged_rows = 0;
   if (!use_matrix_cores(m_batch)) {
     // VALU path: fewer workgroups than tile groups means every wave walks several tiles.
     const int ov_wg = g_override_workgroups.load();
@@ -1123,6 +1382,53 @@ hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr) {
   }
 }
 
+// LDS-staged matrix-core kernel: 2 tiles per workgroup share the activation stage.
+template <int BITS, int QOP, int GPR, int ROUNDS>
+hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
+  const auto kernel = gemv_mfma_lds_kernel<BITS, QOP, GPR, ROUNDS>;
+  if (g.lds > 48 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds);
+    if (e != hipSuccess) return e;
+  }
+  return launch(kernel, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale, g.zero_add, g.n_out, g.k,
+                pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups, g.tail.num_groups,
+                pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+}
+
+template <int BITS, int QOP, int GPR>
+hipError_t launch_mfma_lds_kernel(const GemvLaunch& g, int rounds) {
+  return rounds == 4 ? launch_mfma_lds_kernel_r<BITS, QOP, GPR, 4>(g) : launch_mfma_lds_kernel_r<BITS, QOP, GPR, 8>(g);
+}
+
+template <int BITS, int QOP>
+hipError_t launch_mfma_lds_gpr(const GemvLaunch& g, int gpr, int rounds) {
+  if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
+    return launch_mfma_lds_kernel<BITS, QOP, 1>(g, rounds);
+  } else {
+    switch (gpr) {
+      case 1: return launch_mfma_lds_kernel<BITS, QOP, 1>(g, rounds);
+      case 2: return launch_mfma_lds_kernel<BITS, QOP, 2>(g, rounds);
+      default: return launch_mfma_lds_kernel<BITS, QOP, 4>(g, rounds);
+    }
+  }
+}
+
+hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds) {
+  if (bits == 4) {
+    switch (qop) {
+      case 1: return launch_mfma_lds_gpr<4, 1>(g, gpr, rounds);
+      case 2: return launch_mfma_lds_gpr<4, 2>(g, gpr, rounds);
+      default: return launch_mfma_lds_gpr<4, 3>(g, gpr, rounds);
+    }
+  }
+  switch (qop) {
+    case 1: return launch_mfma_lds_gpr<8, 1>(g, gpr, rounds);
+    case 2: return launch_mfma_lds_gpr<8, 2>(g, gpr, rounds);
+    default: return launch_mfma_lds_gpr<8, 3>(g, gpr, rounds);
+  }
+}
+
 template <int BITS>
 hipError_t launch_dequant(const DequantParams& p, int qop, half_t* out, hipStream_t stream) {
   const long long units = (long long)p.tiles * p.ksteps;
@@ -1183,6 +1489,14 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
     g.x = reinterpret_cast<const half_t*>(x);
     g.tail.y = reinterpret_cast<half_t*>(y);
     g.tail.m_batch = m_batch;
+    if (g.plan.staged_rows != 0) {
+      const int row_stride = step_k(weight_bits) * 2 + 16;
+      g.lds = (size_t)g.plan.split_k * 2 * g.plan.staged_rows * row_stride +
+              (g.plan.split_k > 1 ? (size_t)g.plan.tiles_per_wg * g.plan.split_k * kWave * 4 * sizeof(float) : 0);
+      return launch_mfma_lds(g, weight_bits, quant_op, gpr, g.plan.staged_rows / g.plan.tiles_per_wg) == hipSuccess
+                 ? MGEMV_OK
+                 : MGEMV_ERR_LAUNCH;
+    }
     g.lds = g.plan.split_k == 1 ? 0
                                 : (size_t)g.plan.tiles_per_wg * g.plan.split_k * g.plan.tiles_per_wave * kWave * 4 * sizeof(float);
     return launch_mfma(g, weight_bits, quant_op, gpr) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
@@ -1243,6 +1557,14 @@ int mgemv_set_matrix_core_threshold(int min_m_batch) {
   return MGEMV_OK;
 }
 
+int mgemv_set_matrix_core_variant(int variant) {
+  if (variant != MGEMV_MATRIX_CORE_AUTO && variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND &&
+      variant != MGEMV_MATRIX_CORE_LDS_STAGED)
+    return MGEMV_ERR_SIZE;
+  mgemv::g_matrix_core_variant.store(variant);
+  return MGEMV_OK;
+}
+
 int mgemv_set_dequant_form(int form) {
   if (form != MGEMV_DEQUANT_AUTO && form != MGEMV_DEQUANT_EXACT_INTEGER) return MGEMV_ERR_SIZE;
   mgemv::g_dequant_flags.store(form == MGEMV_DEQUANT_EXACT_INTEGER ? mgemv::kExactIntegerFormOnly : 0);
@@ -1260,7 +1582,7 @@ int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8
   out[2] = lp.split_k;
   out[3] = lp.tiles_per_wg;
   out[4] = lp.steps_per_wave;
-  out[5] = mgemv::use_matrix_cores(m_batch) ? 1 : 0;
+  out[5] = !mgemv::use_matrix_cores(m_batch) ? 0 : lp.staged_rows != 0 ? 2 : 1;
   out[6] = lp.tiles_per_wave;
   out[7] = lp.tiles_in_sequence;
   return MGEMV_OK;

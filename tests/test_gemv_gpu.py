@@ -283,7 +283,7 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     dev = DeviceProblem(prob, gpu)
     y_all = dev.run().copy()
     assert np.array_equal(y_all.view(np.uint16), dev.run().view(np.uint16))
-    assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (1 if m_batch >= 5 else 0)
+    assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (2 if m_batch >= 5 else 0)   # 2: LDS-staged
     single = Problem("rows", 80, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True)
     for b in range(m_batch):
         single.x = prob.x[b:b + 1].copy()
@@ -298,20 +298,30 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
 @pytest.mark.parametrize("bits,qop,g", [(4, SCALE_AND_ZEROS, 128), (4, SCALE_ONLY, 64), (4, PER_COLUMN, 0),
                                         (8, SCALE_AND_ZEROS, 64), (8, PER_COLUMN, 0), (4, SCALE_AND_ZEROS, 160)])
 def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
-    """The same batches through both kernels (threshold forced), ragged shape, every mode."""
+    """The same batches through the two matrix-core kernels (LDS-staged at several k splits, register
+    operand) and the VALU kernel (threshold forced), ragged shape, every mode."""
     n_out, k = 100, 1120 if g in (0, 160) else 1024
     for m_batch in (1, 5, 8, 13, 16):
         prob = Problem(f"mc{bits}{qop}", n_out, k, bits, qop, g, m_batch=m_batch, bias=True)
         dev = DeviceProblem(prob, gpu)
         ref = prob.oracle_gemv(threads=8)
+        results = []
         try:
             mg.set_matrix_core_threshold(1)
-            y_mc = dev.run().copy()
+            for variant, split in ((mg.MATRIX_CORE_LDS_STAGED, 0), (mg.MATRIX_CORE_LDS_STAGED, 1),
+                                   (mg.MATRIX_CORE_LDS_STAGED, 2), (mg.MATRIX_CORE_REGISTER_OPERAND, 0)):
+                mg.set_matrix_core_variant(variant)
+                mg.set_launch_override(split, 0, 0, 0)
+                assert mg.query_launch(n_out, m_batch, k, bits)["matrix_core"] == (2 if variant == mg.MATRIX_CORE_LDS_STAGED else 1)
+                results.append(dev.run().copy())
+                assert np.array_equal(results[-1].view(np.uint16), dev.run().view(np.uint16))   # reproducible
             mg.set_matrix_core_threshold(17)
-            y_valu = dev.run().copy()
+            results.append(dev.run().copy())   # VALU kernel
         finally:
             mg.set_matrix_core_threshold(0)
-        for y in (y_mc, y_valu):
+            mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
+            mg.set_launch_override(0, 0, 0, 0)
+        for y in results:
             _, rel, _ = error_report(y, ref)
             assert rel <= REL_TOL, (m_batch, rel)
 

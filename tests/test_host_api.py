@@ -205,6 +205,8 @@ def test_gemv_argument_checks_return_codes_without_launching():
     assert lib.mgemv_set_launch_override(-1, 0, 0, 0) == 10
     assert lib.mgemv_set_launch_override(0, 0, 3, 0) == 10
     assert lib.mgemv_set_matrix_core_threshold(18) == 8
+    assert lib.mgemv_set_matrix_core_variant(3) == 10 and lib.mgemv_set_matrix_core_variant(0) == 0
+    assert lib.mgemv_set_dequant_form(2) == 10 and lib.mgemv_set_dequant_form(0) == 0
 
 
 def test_adaptor_mirror_rejects_small_groups_like_the_reference():
