@@ -1108,17 +1108,26 @@ std::atomic<int> g_override_split_k{0};
 std::atomic<int> g_override_tiles_per_wg{0};
 std::atomic<int> g_override_tiles_per_wave{0};
 std::atomic<int> g_override_workgroups{0};
-std::atomic<int> g_matrix_core_min_batch{5};  // m_batch from which the matrix-core kernel is used
+std::atomic<int> g_matrix_core_min_batch{0};  // m_batch from which the matrix-core kernels are used; 0 = built-in rule
 std::atomic<int> g_dequant_flags{0};          // kExactIntegerFormOnly or 0
 std::atomic<int> g_matrix_core_variant{MGEMV_MATRIX_CORE_AUTO};
 
-inline bool use_matrix_cores(int m_batch) { return m_batch >= g_matrix_core_min_batch.load(); }
+// Built-in rule, measured: up to 4 activation rows the VALU kernel wins on matrices of up to
+// ~8k units (8192x8192: 12.0 us at 4 rows against 11.8 us, 10.9 against 11.9 at 3); on larger ones
+// the LDS-staged matrix-core kernel already wins at 3 rows (28672x8192: 26.9 us against 31.9 us).
+// From 5 rows the VALU kernel would need a second launch.
+inline bool use_matrix_cores(int m_batch, long long units) {
+  const int forced = g_matrix_core_min_batch.load();
+  if (forced > 0) return m_batch >= forced;
+  return m_batch >= 5 || (m_batch >= 3 && units >= 16384);
+}
 
 struct LaunchPlan {
   int split_k, tiles_per_wg, steps_per_wave, workgroups, wgs_per_xcd, threads;
   int tiles_per_wave;  // 1 on the VALU path; 1, 2 or 4 on the matrix-core path
   int tiles_in_sequence;  // VALU path: most tiles any wave walks one after the other
   int staged_rows;        // LDS-staged matrix-core kernel: 8 or 16 activation rows per stage; 0 = other kernels
+  bool matrix_core;       // one of the two matrix-core kernels (else the VALU kernel)
 };
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -1127,10 +1136,12 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
   const int ov_t = g_override_tiles_per_wave.load();
-  if (use_matrix_cores(m_batch) && g_matrix_core_variant.load() != MGEMV_MATRIX_CORE_REGISTER_OPERAND && tiles >= 2) {
+  const bool mc = use_matrix_cores(m_batch, (long long)tiles * ksteps);
+  if (mc && g_matrix_core_variant.load() != MGEMV_MATRIX_CORE_REGISTER_OPERAND && tiles >= 2) {
     // LDS-staged kernel: two tiles per workgroup share the activation stage; k split until the
     // launch has about 1.5 k waves (measured: 8192x8192 best at 4 k-split waves, 28672x8192 at 1).
     LaunchPlan lp{};
+    lp.matrix_core = true;
     lp.tiles_per_wg = 2;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
@@ -1150,7 +1161,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   // once for all of them.  Measured on 8192 x 8192 (512 tiles): T = 2 is 1.5-1.8x faster than
   // T = 1 at 8-16 activation rows; T = 4 leaves too few waves to cover the load latency.
   int tiles_per_wave = 1;
-  if (use_matrix_cores(m_batch)) {
+  if (mc) {
     tiles_per_wave = tiles >= 256 ? 2 : 1;
     if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
   }
@@ -1163,24 +1174,24 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   //  * more tile groups than that: split as far as the units allow (at most 16 waves) while the
   //    launch stays under ~8k waves, and fall back to two units per wave when that still
   //    leaves >= 4096 waves (8192x8192: 10.6 us at 8 waves vs 11.2 us at 16).
-  const int max_waves = use_matrix_cores(m_batch) ? kMaxWavesPerMfmaWorkgroup
+  const int max_waves = mc ? kMaxWavesPerMfmaWorkgroup
                         : m_batch >= 3            ? kMaxWavesPerWideWorkgroup
                                                   : kMaxWavesPerWorkgroup;
   int split_k;
   if (groups <= 384) {
     split_k = ksteps < 4 ? ksteps : 4;
-    if (use_matrix_cores(m_batch)) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
+    if (mc) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
   } else {
     constexpr int kWaveBudget = 8192;
     split_k = ksteps < max_waves ? ksteps : max_waves;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
-    if (!use_matrix_cores(m_batch) && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
+    if (!mc && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
         (long long)groups * ((split_k + 1) / 2) >= 4096)
       split_k = (split_k + 1) / 2;
   }
   int tiles_per_wg = 1;
   int workgroup_cap = 0;
-  if (!use_matrix_cores(m_batch) && tiles >= kNumCus && ksteps >= 4) {
+  if (!mc && tiles >= kNumCus && ksteps >= 4) {
     // "Exact fit": when the tiles divide (nearly) evenly over the compute units, one workgroup
     // of four waves per compute unit -- one wave per SIMD, all with the same amount of work --
     // beats any over-subscribed launch (8192x8192: 8.7 us against 10.2 us; 28672x8192: 2 %).
@@ -1209,7 +1220,8 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   lp.workgroups = ceil_div(groups, tiles_per_wg);
   lp.tiles_in_sequence = 1;
   lp.staged_rows = 0;
-  if (!use_matrix_cores(m_batch)) {
+  lp.matrix_core = mc;
+  if (!mc) {
     // VALU path: fewer workgroups than tile groups means every wave walks several tiles.
     const int ov_wg = g_override_workgroups.load();
     int cap = ov_wg > 0 ? ov_wg : (workgroup_cap > 0 && ov_sk == 0 && ov_tw == 0) ? workgroup_cap : lp.workgroups;
@@ -1485,7 +1497,7 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.stream = static_cast<hipStream_t>(stream);
   const int gpr = groups_per_run(group_size, weight_bits);
 
-  if (use_matrix_cores(m_batch)) {
+  if (g.plan.matrix_core) {
     g.x = reinterpret_cast<const half_t*>(x);
     g.tail.y = reinterpret_cast<half_t*>(y);
     g.tail.m_batch = m_batch;
@@ -1553,7 +1565,7 @@ int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int ti
 
 int mgemv_set_matrix_core_threshold(int min_m_batch) {
   if (min_m_batch < 0 || min_m_batch > MGEMV_MAX_M_BATCH + 1) return MGEMV_ERR_BATCH;
-  mgemv::g_matrix_core_min_batch.store(min_m_batch == 0 ? 5 : min_m_batch);
+  mgemv::g_matrix_core_min_batch.store(min_m_batch);
   return MGEMV_OK;
 }
 
@@ -1582,7 +1594,7 @@ int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8
   out[2] = lp.split_k;
   out[3] = lp.tiles_per_wg;
   out[4] = lp.steps_per_wave;
-  out[5] = !mgemv::use_matrix_cores(m_batch) ? 0 : lp.staged_rows != 0 ? 2 : 1;
+  out[5] = !lp.matrix_core ? 0 : lp.staged_rows != 0 ? 2 : 1;
   out[6] = lp.tiles_per_wave;
   out[7] = lp.tiles_in_sequence;
   return MGEMV_OK;
