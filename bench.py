@@ -370,7 +370,7 @@ def main():
     value = wl.bytes / (wall / steps) / 1e9
     kernel_us = ev_us
     achieved = wl.bytes / (kernel_us * 1e-6) / 1e9
-    plan = mg.query_launch(wl.n_out, wl.m_batch, wl.k, wl.bits)
+    plan = mg.query_launch(wl.n_out, wl.m_batch, wl.k, wl.bits, wl.k if wl.quant_op == 1 else wl.group)
 
     out = {
         "metric": "HBM GB/s & % of peak, us/call; int4-g128 GEMV M=1, N=K=4096",

@@ -178,11 +178,13 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Which of the two matrix-core kernels serves the small batches:
- *   MGEMV_MATRIX_CORE_AUTO (default)          the LDS-staged kernel wherever the matrix has at least two
- *                                             16-row tiles, else the register-operand kernel;
+ *   MGEMV_MATRIX_CORE_AUTO (default)          the register-operand kernel, one tile per wave, on matrices
+ *                                             of up to 256 16-row tiles with up to 8 activation rows,
+ *                                             else the LDS-staged kernel;
  *   MGEMV_MATRIX_CORE_REGISTER_OPERAND        always the kernel that reads its activation operand from
  *                                             L2 into registers;
- *   MGEMV_MATRIX_CORE_LDS_STAGED              same choice as AUTO (named for symmetry in tests).
+ *   MGEMV_MATRIX_CORE_LDS_STAGED              the LDS-staged kernel wherever the matrix has at least two
+ *                                             tiles.
  * Same results to tolerance either way (the k split, hence the order of the fp32 sums, differs).
  * For tests and measurements; no counterpart in the reference.  Process-wide. */
 enum { MGEMV_MATRIX_CORE_AUTO = 0, MGEMV_MATRIX_CORE_REGISTER_OPERAND = 1, MGEMV_MATRIX_CORE_LDS_STAGED = 2 };
@@ -199,13 +201,41 @@ MGEMV_API int mgemv_set_matrix_core_variant(int variant);
 enum { MGEMV_DEQUANT_AUTO = 0, MGEMV_DEQUANT_EXACT_INTEGER = 1 };
 MGEMV_API int mgemv_set_dequant_form(int form);
 
-/* Reports the geometry mgemv_gemv would use: out[0] = workgroups, out[1] = threads per
+/* Tuned plans: a table keyed on the problem (n_out, k, weight_bits, group_size, m_batch) that
+ * replaces the built-in launch rules for exactly that problem -- the run-time counterpart of
+ * choosing the reference's compile-time ThreadBlockShape / WarpShape / kStages per problem
+ * (mixed_gemv_test.cu:40, 67-70; the 1- vs 2-stage main loops of
+ * gemv/threadblock/default_dq_mma_simt.h:224-234 and 394-404).  group_size = 0 in an entry
+ * matches every group size (an entry for the exact group size wins); per-column problems are
+ * looked up with group_size = k.  The knobs have the meaning of mgemv_set_launch_override
+ * (0 = built-in rule for that knob); `kernel` picks the kernel.  A process-wide override that is
+ * set (mgemv_set_launch_override, _matrix_core_threshold, _matrix_core_variant) takes precedence
+ * over the table.  Setting an existing key replaces it.  Results never depend on the plan beyond
+ * the order of the fp32 partial sums.  Thread-safe. */
+enum {
+  MGEMV_KERNEL_AUTO = 0,
+  MGEMV_KERNEL_VALU = 1,
+  MGEMV_KERNEL_MATRIX_CORE_REGISTER_OPERAND = 2,
+  MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED = 3
+};
+typedef struct mgemv_tuned_plan {
+  int n_out, k, weight_bits, group_size, m_batch; /* key */
+  int kernel;                                     /* MGEMV_KERNEL_* */
+  int split_k_waves, tiles_per_workgroup, tiles_per_wave, max_workgroups;
+} mgemv_tuned_plan;
+MGEMV_API int mgemv_tuned_plan_set(const mgemv_tuned_plan *plan);
+MGEMV_API int mgemv_tuned_plan_clear(void);
+MGEMV_API int mgemv_tuned_plan_count(void);
+
+/* Reports the geometry mgemv_gemv would use for this problem (group_size as passed to mgemv_gemv,
+ * k for per-column problems, 0 to consult only table entries for any group size):
+ * out[0] = workgroups, out[1] = threads per
  * workgroup, out[2] = k-split waves per tile, out[3] = tile sequences per workgroup,
  * out[4] = k steps per wave and tile, out[5] = 0 VALU kernel / 1 matrix-core kernel with the
  * activation operand in registers / 2 LDS-staged matrix-core kernel,
  * out[6] = tiles per wave (matrix-core path), out[7] = most tiles a wave walks one after the
  * other (VALU path). */
-MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8]);
+MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]);
 
 #ifdef __cplusplus
 }

@@ -26,7 +26,15 @@ from .api import (  # noqa: F401
     DEQUANT_AUTO,
     DEQUANT_EXACT_INTEGER,
     unpreprocess_weights,
+    set_tuned_plan,
+    clear_tuned_plans,
+    tuned_plan_count,
+    KERNEL_AUTO,
+    KERNEL_VALU,
+    KERNEL_MATRIX_CORE_REGISTER_OPERAND,
+    KERNEL_MATRIX_CORE_LDS_STAGED,
 )
+from . import autotune  # noqa: F401
 from ._lib import LIB_PATH, MixedGemvError  # noqa: F401
 
 __version__ = "0.1.0"

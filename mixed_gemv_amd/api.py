@@ -235,10 +235,33 @@ def set_dequant_form(form=DEQUANT_AUTO):
     _lib.check(_lib.lib().mgemv_set_dequant_form(int(form)), "set_dequant_form")
 
 
-def query_launch(n_out, m_batch, k, weight_bits=4):
+def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0):
+    """The geometry mgemv_gemv would use (group_size as passed to the GEMV; it only selects tuned plans)."""
     out = (ctypes.c_int * 8)()
-    _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), ctypes.byref(out)),
-               "query_launch")
+    _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size),
+                                             ctypes.byref(out)), "query_launch")
     keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave",
             "tiles_in_sequence")
     return dict(zip(keys, list(out)))
+
+
+KERNEL_AUTO = 0
+KERNEL_VALU = 1
+KERNEL_MATRIX_CORE_REGISTER_OPERAND = 2
+KERNEL_MATRIX_CORE_LDS_STAGED = 3
+
+
+def set_tuned_plan(n_out, k, weight_bits, group_size, m_batch, kernel=KERNEL_AUTO, split_k=0, tiles_per_wg=0,
+                   tiles_per_wave=0, max_workgroups=0):
+    """Installs the launch plan for exactly this problem; see mgemv_tuned_plan_set (group_size 0 = any)."""
+    plan = (ctypes.c_int * 10)(int(n_out), int(k), int(weight_bits), int(group_size), int(m_batch), int(kernel),
+                               int(split_k), int(tiles_per_wg), int(tiles_per_wave), int(max_workgroups))
+    _lib.check(_lib.lib().mgemv_tuned_plan_set(ctypes.byref(plan)), "set_tuned_plan")
+
+
+def clear_tuned_plans():
+    _lib.check(_lib.lib().mgemv_tuned_plan_clear(), "clear_tuned_plans")
+
+
+def tuned_plan_count():
+    return int(_lib.lib().mgemv_tuned_plan_count())

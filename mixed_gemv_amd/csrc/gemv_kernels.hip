@@ -14,6 +14,9 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <map>
+#include <mutex>
+#include <tuple>
 
 #include "device_math.h"
 #include "mixed_gemv.h"
@@ -1112,12 +1115,43 @@ std::atomic<int> g_matrix_core_min_batch{0};  // m_batch from which the matrix-c
 std::atomic<int> g_dequant_flags{0};          // kExactIntegerFormOnly or 0
 std::atomic<int> g_matrix_core_variant{MGEMV_MATRIX_CORE_AUTO};
 
+// What steers plan_launch besides the shape: zeros mean "built-in rule".
+struct PlanKnobs {
+  int split_k = 0, tiles_per_wg = 0, tiles_per_wave = 0, workgroups = 0;
+  int matrix_core_min_batch = 0;
+  int matrix_core_variant = MGEMV_MATRIX_CORE_AUTO;
+};
+
+// Tuned plans by problem: (n_out, k, weight bits, group size or 0 for any, m_batch) -> knobs.
+using PlanKey = std::tuple<int, int, int, int, int>;
+std::mutex g_tuned_mutex;
+std::map<PlanKey, PlanKnobs> g_tuned_plans;
+std::atomic<int> g_tuned_count{0};  // lets the launch path skip the lock while the table is empty
+
+// Process-wide overrides win over the table (they are what a tuner sweeps); then an entry for
+// exactly this group size, then one for any group size, then the built-in rules.
+PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
+  PlanKnobs kn;
+  kn.split_k = g_override_split_k.load();
+  kn.tiles_per_wg = g_override_tiles_per_wg.load();
+  kn.tiles_per_wave = g_override_tiles_per_wave.load();
+  kn.workgroups = g_override_workgroups.load();
+  kn.matrix_core_min_batch = g_matrix_core_min_batch.load();
+  kn.matrix_core_variant = g_matrix_core_variant.load();
+  const bool overridden = kn.split_k || kn.tiles_per_wg || kn.tiles_per_wave || kn.workgroups ||
+                          kn.matrix_core_min_batch || kn.matrix_core_variant != MGEMV_MATRIX_CORE_AUTO;
+  if (overridden || g_tuned_count.load() == 0) return kn;
+  std::lock_guard<std::mutex> lock(g_tuned_mutex);
+  auto it = g_tuned_plans.find(PlanKey{n_out, k, bits, group_size, m_batch});
+  if (it == g_tuned_plans.end() && group_size != 0) it = g_tuned_plans.find(PlanKey{n_out, k, bits, 0, m_batch});
+  return it == g_tuned_plans.end() ? kn : it->second;
+}
+
 // Built-in rule, measured: up to 4 activation rows the VALU kernel wins on matrices of up to
 // ~8k units (8192x8192: 12.0 us at 4 rows against 11.8 us, 10.9 against 11.9 at 3); on larger ones
 // the LDS-staged matrix-core kernel already wins at 3 rows (28672x8192: 26.9 us against 31.9 us).
 // From 5 rows the VALU kernel would need a second launch.
-inline bool use_matrix_cores(int m_batch, long long units) {
-  const int forced = g_matrix_core_min_batch.load();
+inline bool use_matrix_cores(int m_batch, long long units, int forced) {
   if (forced > 0) return m_batch >= forced;
   return m_batch >= 5 || (m_batch >= 3 && units >= 16384);
 }
@@ -1132,21 +1166,28 @@ struct LaunchPlan {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
+LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs& knobs) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
-  const int ov_sk = g_override_split_k.load(), ov_tw = g_override_tiles_per_wg.load();
-  const int ov_t = g_override_tiles_per_wave.load();
-  const bool mc = use_matrix_cores(m_batch, (long long)tiles * ksteps);
-  if (mc && g_matrix_core_variant.load() != MGEMV_MATRIX_CORE_REGISTER_OPERAND && tiles >= 2) {
-    // LDS-staged kernel: two tiles per workgroup share the activation stage; k split until the
-    // launch has about 1.5 k waves (measured: 8192x8192 best at 4 k-split waves, 28672x8192 at 1).
+  const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
+  const int ov_t = knobs.tiles_per_wave;
+  const bool mc = use_matrix_cores(m_batch, (long long)tiles * ksteps, knobs.matrix_core_min_batch);
+  // Up to 256 tiles and 8 rows the register-operand kernel with one tile per wave wins: a lane of
+  // a row past m_batch loads nothing there, and no barrier ties the waves of a workgroup together
+  // (1024x2048, 5 rows: 3.6 us against 4.6 us; 4096x11008: 10.2 against 13.3; 4096x4096, 8 rows: 6.3
+  // against 6.7; at 16 rows, or from 384 tiles, the LDS-staged kernel is level or ahead).
+  const bool small_problem = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && tiles <= 256 && m_batch <= 8;
+  if (mc && knobs.matrix_core_variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND && !small_problem && tiles >= 2) {
+    // LDS-staged kernel: two tiles per workgroup share the activation stage; k split as long as
+    // the launch stays within 2048 waves (measured: 8192x8192 best at 4 k-split waves, 11008x4096
+    // at 2 -- 11.4 us against 14.2 us at 4 with 16 rows, whose 133 KB of stages would leave one
+    // workgroup per compute unit for 344 workgroups --, 28672x8192 at 1).
     LaunchPlan lp{};
     lp.matrix_core = true;
     lp.tiles_per_wg = 2;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
     int split = 1;
-    while (split < 4 && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split < 1536) split *= 2;
+    while (split < 4 && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 2048) split *= 2;
     if (ov_sk > 0) split = ov_sk > 4 ? 4 : ov_sk;
     if (split > ksteps) split = ksteps;
     lp.steps_per_wave = ceil_div(ksteps, split);
@@ -1162,7 +1203,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   // T = 1 at 8-16 activation rows; T = 4 leaves too few waves to cover the load latency.
   int tiles_per_wave = 1;
   if (mc) {
-    tiles_per_wave = tiles >= 256 ? 2 : 1;
+    tiles_per_wave = tiles >= 256 && !small_problem ? 2 : 1;
     if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
   }
   const int groups = ceil_div(tiles, tiles_per_wave);
@@ -1223,7 +1264,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch) {
   lp.matrix_core = mc;
   if (!mc) {
     // VALU path: fewer workgroups than tile groups means every wave walks several tiles.
-    const int ov_wg = g_override_workgroups.load();
+    const int ov_wg = knobs.workgroups;
     int cap = ov_wg > 0 ? ov_wg : (workgroup_cap > 0 && ov_sk == 0 && ov_tw == 0) ? workgroup_cap : lp.workgroups;
     if (cap < lp.workgroups) lp.workgroups = cap;
     const int rows = m_batch < kMaxValuBatch ? m_batch : kMaxValuBatch;
@@ -1477,7 +1518,7 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.n_out = n_out;
   g.k = k;
   g.group_size = group_size;
-  g.plan = plan_launch(n_out, k, weight_bits, m_batch);
+  g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs_for(n_out, k, weight_bits, group_size, m_batch));
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
@@ -1583,12 +1624,62 @@ int mgemv_set_dequant_form(int form) {
   return MGEMV_OK;
 }
 
-int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int out[8]) {
-  if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
+namespace {
+int check_tuned_key(int n_out, int k, int weight_bits, int group_size, int m_batch) {
   if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
   if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
+  if (group_size < 0) return MGEMV_ERR_GROUP_SIZE;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
-  const mgemv::LaunchPlan lp = mgemv::plan_launch(n_out, k, weight_bits, m_batch);
+  return MGEMV_OK;
+}
+}  // namespace
+
+int mgemv_tuned_plan_set(const mgemv_tuned_plan* plan) {
+  if (plan == nullptr) return MGEMV_ERR_NULL_POINTER;
+  const int st = check_tuned_key(plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch);
+  if (st != MGEMV_OK) return st;
+  if (plan->split_k_waves < 0 || plan->tiles_per_workgroup < 0 || plan->max_workgroups < 0) return MGEMV_ERR_SIZE;
+  const int t = plan->tiles_per_wave;
+  if (t != 0 && t != 1 && t != 2 && t != 4) return MGEMV_ERR_SIZE;
+  mgemv::PlanKnobs kn;
+  kn.split_k = plan->split_k_waves;
+  kn.tiles_per_wg = plan->tiles_per_workgroup;
+  kn.tiles_per_wave = t;
+  kn.workgroups = plan->max_workgroups;
+  switch (plan->kernel) {
+    case MGEMV_KERNEL_AUTO: break;
+    case MGEMV_KERNEL_VALU: kn.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1; break;
+    case MGEMV_KERNEL_MATRIX_CORE_REGISTER_OPERAND:
+      kn.matrix_core_min_batch = 1;
+      kn.matrix_core_variant = MGEMV_MATRIX_CORE_REGISTER_OPERAND;
+      break;
+    case MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED:
+      kn.matrix_core_min_batch = 1;
+      kn.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
+      break;
+    default: return MGEMV_ERR_SIZE;
+  }
+  std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);
+  mgemv::g_tuned_plans[mgemv::PlanKey{plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch}] = kn;
+  mgemv::g_tuned_count.store((int)mgemv::g_tuned_plans.size());
+  return MGEMV_OK;
+}
+
+int mgemv_tuned_plan_clear(void) {
+  std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);
+  mgemv::g_tuned_plans.clear();
+  mgemv::g_tuned_count.store(0);
+  return MGEMV_OK;
+}
+
+int mgemv_tuned_plan_count(void) { return mgemv::g_tuned_count.load(); }
+
+int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]) {
+  if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
+  const int st = check_tuned_key(n_out, k, weight_bits, group_size, m_batch);
+  if (st != MGEMV_OK) return st;
+  const mgemv::LaunchPlan lp = mgemv::plan_launch(n_out, k, weight_bits, m_batch,
+                                                  mgemv::knobs_for(n_out, k, weight_bits, group_size, m_batch));
   out[0] = lp.wgs_per_xcd * mgemv::kNumXcd;
   out[1] = lp.threads;
   out[2] = lp.split_k;

@@ -240,6 +240,53 @@ def test_split_k_invariance_and_determinism(gpu):
             assert np.array_equal(results[same[0]].view(np.uint16), results[other].view(np.uint16)), (same[0], other)
 
 
+def test_tuned_plan_equals_the_same_override_bit_for_bit(gpu):
+    from mixed_gemv_amd import autotune
+    prob = Problem("tuned", 192, 4096, 4, SCALE_AND_ZEROS, 128, bias=True, x_dist="normal")
+    dev = DeviceProblem(prob, gpu)
+    autotune.clear()
+    try:
+        builtin = dev.run().copy()
+        for sk, tw, cap in ((8, 2, 0), (2, 1, 3)):
+            mg.set_launch_override(sk, tw, 0, cap)
+            forced = dev.run().copy()
+            mg.set_launch_override(0, 0, 0, 0)
+            mg.set_tuned_plan(192, 4096, 4, 128, 1, kernel=mg.KERNEL_VALU, split_k=sk, tiles_per_wg=tw, max_workgroups=cap)
+            tuned = dev.run().copy()
+            assert np.array_equal(forced.view(np.uint16), tuned.view(np.uint16))
+        autotune.clear()
+        assert np.array_equal(builtin.view(np.uint16), dev.run().view(np.uint16))
+    finally:
+        autotune.clear()
+        mg.set_launch_override(0, 0, 0, 0)
+
+
+@pytest.mark.parametrize("m_batch", [1, 6])
+def test_tuner_measures_installs_and_keeps_parity(gpu, m_batch):
+    """The tuner on a small problem: every candidate it keeps is a distinct geometry, the overrides
+    it sweeps are gone afterwards, and whatever it installed still meets the parity bar."""
+    from mixed_gemv_amd import autotune
+    prob = Problem("tuner", 1024, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=m_batch, bias=True)
+    autotune.clear()
+    try:
+        before = mg.query_launch(1024, m_batch, 2048, 4, 128)
+        lines = []
+        res = autotune.tune(1024, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=m_batch, bias=True, launches=64, rounds=1,
+                            min_gain=0.0, cold_bytes=8 << 20, log=lines.append)
+        print("\n".join(lines), flush=True)
+        assert len(res["measurements"]) >= 4 and all(us > 0 for us, _ in res["measurements"])
+        assert res["entry"] is None or res["entry"]["us"] < res["entry"]["builtin_us"]
+        after = mg.query_launch(1024, m_batch, 2048, 4, 128)
+        if res["entry"] is None:
+            assert after == before and mg.tuned_plan_count() == 0
+        else:
+            assert after == res["best_geometry"] and mg.tuned_plan_count() == 1
+        assert mg.query_launch(2048, m_batch, 2048, 4, 128) == mg.query_launch(2048, m_batch, 2048, 4, 0)
+        check(prob, gpu, dequant=False)
+    finally:
+        autotune.clear()
+
+
 WALKS = [
     # tag, n_out, k, bits, quant_op, group, m_batch, bias
     ("w_i4_sz_g64", 208, 2048, 4, SCALE_AND_ZEROS, 64, 1, True),     # two groups per lane run
@@ -274,7 +321,7 @@ def test_tile_walks_match_one_tile_per_wave(gpu, cfg):
         mg.set_launch_override(0, 0, 0, 0)
 
 
-@pytest.mark.parametrize("m_batch", [4, 11])
+@pytest.mark.parametrize("m_batch", [4, 7, 11])
 def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     """Rows of a batch are independent GEMVs.  Up to 4 rows the VALU kernel adds every row in
     the single-row order (bit-identical); from 5 rows the matrix-core kernel takes over, whose
@@ -283,7 +330,9 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     dev = DeviceProblem(prob, gpu)
     y_all = dev.run().copy()
     assert np.array_equal(y_all.view(np.uint16), dev.run().view(np.uint16))
-    assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (2 if m_batch >= 5 else 0)   # 2: LDS-staged
+    assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (0 if m_batch < 5 else 1 if m_batch <= 8 else 2)
+    assert mg.query_launch(80, 7, 2048, 4)["matrix_core"] == 1   # few tiles, <= 8 rows: register operand
+    assert mg.query_launch(8192, 7, 2048, 4)["matrix_core"] == 2
     single = Problem("rows", 80, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True)
     for b in range(m_batch):
         single.x = prob.x[b:b + 1].copy()

@@ -199,14 +199,71 @@ def test_gemv_argument_checks_return_codes_without_launching():
     # per-column mode ignores group_size entirely (mixed_gemv_test.cu:142-143): 16 would be rejected otherwise
     assert lib.mgemv_dequantize(p, p, None, None, 64, 512, 16, 1, 4, None) == 1
     out = (ctypes.c_int * 8)()
-    assert lib.mgemv_query_launch(4096, 1, 4096, 4, ctypes.byref(out)) == 0
+    assert lib.mgemv_query_launch(4096, 1, 4096, 4, 128, ctypes.byref(out)) == 0
     assert out[0] % 8 == 0 and out[1] % 64 == 0 and out[2] * out[4] >= 8
-    assert lib.mgemv_query_launch(4096, 1, 4096, 3, ctypes.byref(out)) == 7
+    assert lib.mgemv_query_launch(4096, 1, 4096, 3, 128, ctypes.byref(out)) == 7
+    assert lib.mgemv_query_launch(4096, 1, 4096, 4, -1, ctypes.byref(out)) == 5
     assert lib.mgemv_set_launch_override(-1, 0, 0, 0) == 10
     assert lib.mgemv_set_launch_override(0, 0, 3, 0) == 10
     assert lib.mgemv_set_matrix_core_threshold(18) == 8
     assert lib.mgemv_set_matrix_core_variant(3) == 10 and lib.mgemv_set_matrix_core_variant(0) == 0
     assert lib.mgemv_set_dequant_form(2) == 10 and lib.mgemv_set_dequant_form(0) == 0
+
+
+def test_tuned_plan_table_steers_exactly_its_problem(tmp_path):
+    from mixed_gemv_amd import autotune
+    autotune.clear()
+    try:
+        builtin = mg.query_launch(4096, 1, 4096, 4, 128)
+        other = mg.query_launch(8192, 1, 8192, 4, 64)
+        mg.set_tuned_plan(4096, 4096, 4, 128, 1, kernel=mg.KERNEL_VALU, split_k=8, tiles_per_wg=2)
+        assert mg.tuned_plan_count() == 1
+        tuned = mg.query_launch(4096, 1, 4096, 4, 128)
+        assert (tuned["split_k"], tuned["tiles_per_wg"], tuned["matrix_core"]) == (8, 2, 0) and tuned != builtin
+        # other group size, batch size, weight width or shape: untouched
+        assert mg.query_launch(4096, 1, 4096, 4, 64) == builtin
+        assert mg.query_launch(4096, 2, 4096, 4, 128) == mg.query_launch(4096, 2, 4096, 4, 0)
+        assert mg.query_launch(8192, 1, 8192, 4, 64) == other
+        # an entry for any group size; the exact one still wins where it exists
+        mg.set_tuned_plan(4096, 4096, 4, 0, 1, kernel=mg.KERNEL_VALU, split_k=2, tiles_per_wg=1)
+        assert mg.query_launch(4096, 1, 4096, 4, 64)["split_k"] == 2
+        assert mg.query_launch(4096, 1, 4096, 4, 128)["split_k"] == 8
+        # replacing a key keeps the count; kernel choice for a small batch
+        mg.set_tuned_plan(4096, 4096, 4, 128, 1, kernel=mg.KERNEL_VALU, split_k=4, tiles_per_wg=1)
+        assert mg.tuned_plan_count() == 2 and mg.query_launch(4096, 1, 4096, 4, 128)["split_k"] == 4
+        mg.set_tuned_plan(4096, 4096, 4, 128, 4, kernel=mg.KERNEL_MATRIX_CORE_LDS_STAGED)
+        assert mg.query_launch(4096, 4, 4096, 4, 128)["matrix_core"] == 2
+        mg.set_tuned_plan(4096, 4096, 4, 128, 8, kernel=mg.KERNEL_MATRIX_CORE_REGISTER_OPERAND, tiles_per_wave=2)
+        q = mg.query_launch(4096, 8, 4096, 4, 128)
+        assert q["matrix_core"] == 1 and q["tiles_per_wave"] == 2
+        mg.set_tuned_plan(4096, 4096, 4, 128, 16, kernel=mg.KERNEL_VALU)
+        assert mg.query_launch(4096, 16, 4096, 4, 128)["matrix_core"] == 0
+        # a process-wide override takes precedence over the table
+        mg.set_launch_override(8, 1, 0, 0)
+        assert mg.query_launch(4096, 1, 4096, 4, 128)["split_k"] == 8
+        mg.set_launch_override(0, 0, 0, 0)
+        assert mg.query_launch(4096, 1, 4096, 4, 128)["split_k"] == 4
+        # the JSON table carries entries from one process to the next
+        autotune.install(dict(n_out=11008, k=4096, weight_bits=4, group_size=128, m_batch=1, kernel=mg.KERNEL_VALU,
+                              split_k=2, tiles_per_wg=2, max_workgroups=256))
+        want = mg.query_launch(11008, 1, 4096, 4, 128)
+        autotune.save_table(tmp_path / "plans.json")
+        autotune.clear()
+        assert mg.tuned_plan_count() == 0 and mg.query_launch(4096, 1, 4096, 4, 128) == builtin
+        assert autotune.load_table(tmp_path / "plans.json") == 1
+        assert mg.query_launch(11008, 1, 4096, 4, 128) == want
+        # argument checks
+        for bad, code in ((dict(weight_bits=5), 7), (dict(n_out=0), 10), (dict(group_size=-1), 5), (dict(m_batch=0), 8),
+                          (dict(m_batch=17), 8), (dict(kernel=4), 10), (dict(tiles_per_wave=3), 10), (dict(split_k=-1), 10)):
+            args = dict(n_out=64, k=512, weight_bits=4, group_size=128, m_batch=1)
+            args.update(bad)
+            with pytest.raises(MixedGemvError) as ei:
+                mg.set_tuned_plan(**args)
+            assert ei.value.status == code
+        assert _lib.lib().mgemv_tuned_plan_set(None) == 1
+    finally:
+        autotune.clear()
+        mg.set_launch_override(0, 0, 0, 0)
 
 
 def test_adaptor_mirror_rejects_small_groups_like_the_reference():
