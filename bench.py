@@ -69,10 +69,13 @@ def algorithmic_bytes(n_out, k, bits, quant_op, group, m_batch, bias):
 class Workload:
     """Builds the rotating operand sets of one workload directly in HBM (torch is the allocator)."""
 
-    def __init__(self, name, device, m_batch=None, seed=1234, min_sets=None):
+    def __init__(self, name, device, m_batch=None, seed=1234, min_sets=None, element="f16"):
         import numpy as np
         import torch
         import mixed_gemv_amd as mg
+
+        self.element = element
+        dt = torch.bfloat16 if element == "bf16" else torch.half   # activations, scales, zeros, bias, outputs
 
         (self.n_out, self.k, self.bits, self.quant_op, self.group, mb, self.has_bias, xdist, srange,
          self.description) = WORKLOADS[name]
@@ -111,13 +114,13 @@ class Workload:
             w = carve(base, w_bytes, torch.uint8, (w_bytes,))
             w.copy_(torch.from_numpy(pre))
             self.w.append(w)
-            sc = (torch.rand((groups, self.n_out), generator=gen) * (srange[1] - srange[0]) + srange[0]).half()
-            sdev = carve(base + align(w_bytes), s_bytes, torch.half, (groups, self.n_out))
+            sc = (torch.rand((groups, self.n_out), generator=gen) * (srange[1] - srange[0]) + srange[0]).to(dt)
+            sdev = carve(base + align(w_bytes), s_bytes, dt, (groups, self.n_out))
             sdev.copy_(sc)
             self.s.append(sdev)
             if self.quant_op == 3:
-                zz = (torch.rand((groups, self.n_out), generator=gen) * 0.1 - 0.05).half()
-                zdev = carve(base + align(w_bytes) + align(s_bytes), s_bytes, torch.half, (groups, self.n_out))
+                zz = (torch.rand((groups, self.n_out), generator=gen) * 0.1 - 0.05).to(dt)
+                zdev = carve(base + align(w_bytes) + align(s_bytes), s_bytes, dt, (groups, self.n_out))
                 zdev.copy_(zz)
                 self.z.append(zdev)
             else:
@@ -126,9 +129,9 @@ class Workload:
             x = torch.rand((self.m_batch, self.k), generator=gen) * 2 - 1
         else:
             x = torch.randn((self.m_batch, self.k), generator=gen).clamp_(-4, 4)
-        self.x = x.half().to(device)
-        self.bias = (torch.rand((self.n_out,), generator=gen) * 0.2 - 0.1).half().to(device) if self.has_bias else None
-        self.y = torch.zeros((self.m_batch, self.n_out), dtype=torch.half, device=device)
+        self.x = x.to(dt).to(device)
+        self.bias = (torch.rand((self.n_out,), generator=gen) * 0.2 - 0.1).to(dt).to(device) if self.has_bias else None
+        self.y = torch.zeros((self.m_batch, self.n_out), dtype=dt, device=device)
         self.np = np
         self.mg = mg
 
@@ -137,7 +140,7 @@ class Workload:
             return self.launch_batched(i)
         j = i % self.sets
         self.mg.device_gemv(self.w[j], self.x, self.s[j], self.z[j], self.bias, self.y, 1, self.n_out, self.m_batch,
-                            self.k, self.group, self.quant_op, self.bits)
+                            self.k, self.group, self.quant_op, self.bits, element=self.element)
 
     def enable_batched(self, batch):
         """Later launches run `batch` consecutive buffer sets as ONE batched launch (the reference's
@@ -146,14 +149,15 @@ class Workload:
         import torch
         self.batch = batch
         self.set_stride = (self.w[1].data_ptr() - self.w[0].data_ptr()) if self.sets > 1 else 0
-        self.y_batched = torch.zeros((batch, self.m_batch, self.n_out), dtype=torch.half, device=self.y.device)
+        self.y_batched = torch.zeros((batch, self.m_batch, self.n_out), dtype=self.y.dtype, device=self.y.device)
 
     def launch_batched(self, i):
         b = self.batch
         j = (i % (self.sets // b)) * b
         self.mg.device_gemv(self.w[j], self.x, self.s[j], self.z[j], self.bias, self.y_batched, b, self.n_out,
                             self.m_batch, self.k, self.group, self.quant_op, self.bits,
-                            batch_strides=(self.set_stride, 0, self.set_stride // 2, 0, self.m_batch * self.n_out))
+                            batch_strides=(self.set_stride, 0, self.set_stride // 2, 0, self.m_batch * self.n_out),
+                            element=self.element)
 
     def host_operands(self, j=0):
         np = self.np
@@ -331,9 +335,10 @@ def main():
     ap.add_argument("--launch", default="graph", choices=["graph", "stream"],
                     help="graph: the steps are replayed from a captured HIP graph (one kernel node per step, one "
                          "rotation of the buffer sets per replay); stream: one host launch per step")
-    ap.add_argument("--extra", default="c5,nsx8,nsx16",
+    ap.add_argument("--extra", default="c5,nsx8,nsx16,ns:bf16,c5:bf16",
                     help="comma list of further workloads reported under 'other_workloads' ('' = none); "
-                         "'<name>x<B>' runs B problems per launch through the batched entry point")
+                         "'<name>x<B>' runs B problems per launch through the batched entry point, "
+                         "'<name>:bf16' runs the bfloat16 entry point")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / oracle check")
     ap.add_argument("--no-warm-cache", action="store_true",
                     help="skip the warm-cache and launch-floor side measurements (keeps a kernel trace to the cold launches)")
@@ -430,14 +435,16 @@ def main():
     others = {}
     for name in [n for n in args.extra.split(",") if n and n != args.workload]:
         # "<workload>x<B>": B problems per launch through the batched entry point
-        base, _, batch = name.partition("x")
+        base, _, element = name.partition(":")
+        base, _, batch = base.partition("x")
         batch = int(batch) if batch else 1
-        w2 = Workload(base, device, min_sets=5 * batch if batch > 1 else None)
+        w2 = Workload(base, device, min_sets=5 * batch if batch > 1 else None, element=element or "f16")
         if batch > 1:
             w2.enable_batched(batch)
         wall2, ev2, st2, _ = time_workload(w2, max(200, args.steps // (8 * batch)), max(20, args.warmup // 4),
                                            use_graph=(args.launch == "graph"))
-        others[name] = {"workload": w2.description + (f", {batch} independent problems per launch" if batch > 1 else ""),
+        others[name] = {"workload": w2.description + (f", {batch} independent problems per launch" if batch > 1 else "")
+                        + (", bfloat16 activations / scales / outputs" if element == "bf16" else ""),
                         "us_per_call": round(wall2 * 1e6 / st2, 3),
                         "us_per_problem": round(wall2 * 1e6 / st2 / batch, 3),
                         "value_GBps": round(batch * w2.bytes / (wall2 / st2) / 1e9, 1),

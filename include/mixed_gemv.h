@@ -3,7 +3,8 @@
  *
  *     y[b][n] = fp16( sum_k dequant(W)[n][k] * x[b][k]  (+ bias[n]) )
  *
- * int4 or int8 weights, fp16 activations, fp32 accumulation, fp16 output.  The entry
+ * int4 or int8 weights, fp16 (or, in the _bf16 entry points, bfloat16) activations, fp32
+ * accumulation, output in the activation type.  The entry
  * points below are what a binding of JJXiangJiaoJun/mixed_gemv's C++ call sites needs; each
  * one names the reference interface it stands in for.  Dimension names follow the model
  * view: n_out = output features (the reference's M), k = reduction length, m_batch =
@@ -200,6 +201,31 @@ MGEMV_API int mgemv_set_matrix_core_variant(int variant);
  * For tests and measurements.  Process-wide. */
 enum { MGEMV_DEQUANT_AUTO = 0, MGEMV_DEQUANT_EXACT_INTEGER = 1 };
 MGEMV_API int mgemv_set_dequant_form(int form);
+
+/* bfloat16 variants: activations, scales, additive zeros, bias and outputs are bfloat16 bit
+ * patterns (the upper 16 bits of a binary32); everything else -- weights, layouts, argument
+ * meaning, status codes -- is as in the entry point of the same name without the suffix.
+ * They instantiate the reference's templates with ElementB = ElementScale = ElementOutput =
+ * cutlass::bfloat16_t: the converters of gemv/interleaved_numeric_conversion.h:130-183 (int8)
+ * and :340-401 (int4) followed by the dequantiser of gemv/warp/warp_dequantizer.h:52-59, 86-92 --
+ * an instantiation the reference itself still rejects at compile time
+ * (gemv/threadblock/default_dq_mma_simt.h:133-134).  Dequantisation is a bf16 multiply and a bf16
+ * add, each rounded to nearest even; accumulation is fp32; the output is rounded once to bf16.
+ * Every m_batch runs on the VALU kernel (groups of 4 activation rows per launch). */
+MGEMV_API int mgemv_gemv_bf16(const void *weights, const uint16_t *x, const uint16_t *scale,
+                              const uint16_t *zero_add, const uint16_t *bias, uint16_t *y, int n_out, int m_batch,
+                              int k, int group_size, int quant_op, int weight_bits, void *stream);
+MGEMV_API int mgemv_gemv_batched_bf16(const void *weights, const uint16_t *x, const uint16_t *scale,
+                                      const uint16_t *zero_add, const uint16_t *bias, uint16_t *y, int batch_count,
+                                      int n_out, int m_batch, int k, int group_size, int quant_op, int weight_bits,
+                                      int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
+                                      int64_t stride_bias, int64_t stride_y, void *stream);
+MGEMV_API int mgemv_dequantize_bf16(const void *weights, const uint16_t *scale, const uint16_t *zero_add,
+                                    uint16_t *out, int n_out, int k, int group_size, int quant_op, int weight_bits,
+                                    void *stream);
+/* ZeroPointPreprocessor<bfloat16_t,int8_t>::neg_zero_point_multiplies_scale (utils/preprocess.h:94-101):
+ * out[i] = bf16(-zeros[i]) * scales[i], one bf16 multiply. */
+MGEMV_API int mgemv_fold_zero_points_bf16(uint16_t *out, const uint16_t *scales, const int8_t *zeros, size_t n);
 
 /* Tuned plans: a table keyed on the problem (n_out, k, weight_bits, group_size, m_batch) that
  * replaces the built-in launch rules for exactly that problem -- the run-time counterpart of

@@ -28,6 +28,11 @@ SIGNATURES = {
     "mgemv_gemv_batched": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 7
                            + [_c.c_int64] * 5 + [_vp]),
     "mgemv_dequantize": (_c.c_int, [_vp, _u16p, _u16p, _u16p] + [_c.c_int] * 5 + [_vp]),
+    "mgemv_gemv_bf16": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 6 + [_vp]),
+    "mgemv_gemv_batched_bf16": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 7
+                                + [_c.c_int64] * 5 + [_vp]),
+    "mgemv_dequantize_bf16": (_c.c_int, [_vp, _u16p, _u16p, _u16p] + [_c.c_int] * 5 + [_vp]),
+    "mgemv_fold_zero_points_bf16": (_c.c_int, [_u16p, _u16p, _vp, _c.c_size_t]),
     "mgemv_set_launch_override": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int, _c.c_int]),
     "mgemv_set_matrix_core_threshold": (_c.c_int, [_c.c_int]),
     "mgemv_set_dequant_form": (_c.c_int, [_c.c_int]),

@@ -51,6 +51,17 @@ def _dev_ptr(t):
     raise TypeError(f"cannot take a device address from {type(t)!r}")
 
 
+def _is_bf16(element, probe):
+    """element: "f16", "bf16" or None = take it from the dtype of a torch tensor operand (the
+    reference's ElementB / ElementScale / ElementOutput template arguments)."""
+    if element is None:
+        dtype = getattr(probe, "dtype", None)
+        return dtype is not None and str(dtype) == "torch.bfloat16"
+    if element not in ("f16", "bf16"):
+        raise ValueError("element must be 'f16', 'bf16' or None")
+    return element == "bf16"
+
+
 def _stream_ptr(stream):
     if stream is None:
         import torch
@@ -87,16 +98,20 @@ class ZeroPointPreprocessor:
     """utils/preprocess.h:88-102"""
 
     @staticmethod
-    def neg_zero_point_multiplies_scale(scales, zeros):
+    def neg_zero_point_multiplies_scale(scales, zeros, element="f16"):
+        """element="bf16": scales and result are bfloat16 bit patterns in uint16 arrays."""
         s = np.ascontiguousarray(scales)
-        if s.dtype == np.float16:
+        if s.dtype == np.float16 and element == "f16":
             s = s.view(np.uint16)
         if s.dtype != np.uint16:
-            raise TypeError("scales must be float16 (or their uint16 bit patterns)")
+            raise TypeError("scales must be float16 (or uint16 bit patterns of the element type)")
         z = np.ascontiguousarray(zeros, dtype=np.int8)
         if z.size != s.size:
             raise ValueError("scales and zeros differ in size")
         out = np.empty(s.shape, dtype=np.uint16)
+        if _is_bf16(element, None):
+            _lib.check(_lib.lib().mgemv_fold_zero_points_bf16(_host_ptr(out), _host_ptr(s), _host_ptr(z), s.size), "fold")
+            return out
         _lib.check(_lib.lib().mgemv_fold_zero_points(_host_ptr(out), _host_ptr(s), _host_ptr(z), s.size), "fold")
         return out.view(np.float16)
 
@@ -141,21 +156,25 @@ def unpreprocess_weights(preprocessed, shape, quant_type=QuantType.W4_A16):
 
 def device_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, B, M, N, K, group_size,
                 quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, stream=None,
-                batch_strides=None):
+                batch_strides=None, element=None):
     """mixed_gemv_test.cu:124-165.  Reference letters: M = output features, N = activation
     rows, K = reduction, B = batch count.  ptr_A is the PREPROCESSED weight buffer,
     ptr_zero_point the folded fp16 term -z*s, ptr_C an optional fp16 bias.  The quant mode is
-    a run-time argument (a compile-time constant in the reference)."""
+    a run-time argument (a compile-time constant in the reference).  element: "f16" / "bf16" for
+    every 16-bit operand; None takes it from ptr_B when that is a torch tensor, else fp16."""
+    bf16 = _is_bf16(element, ptr_B)
+    gemv = _lib.lib().mgemv_gemv_bf16 if bf16 else _lib.lib().mgemv_gemv
+    gemv_batched = _lib.lib().mgemv_gemv_batched_bf16 if bf16 else _lib.lib().mgemv_gemv_batched
     if B == 1 and not batch_strides:
-        st = _lib.lib().mgemv_gemv(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point),
+        st = gemv(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point),
                                    _dev_ptr(ptr_C), _dev_ptr(ptr_D), int(M), int(N), int(K), int(group_size),
                                    int(quant_op), int(weight_bits), _stream_ptr(stream))
     else:
         sa, sb, ss, sc, sd = batch_strides or (0, 0, 0, 0, 0)
-        st = _lib.lib().mgemv_gemv_batched(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale),
-                                           _dev_ptr(ptr_zero_point), _dev_ptr(ptr_C), _dev_ptr(ptr_D), int(B), int(M),
-                                           int(N), int(K), int(group_size), int(quant_op), int(weight_bits),
-                                           int(sa), int(sb), int(ss), int(sc), int(sd), _stream_ptr(stream))
+        st = gemv_batched(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale),
+                          _dev_ptr(ptr_zero_point), _dev_ptr(ptr_C), _dev_ptr(ptr_D), int(B), int(M),
+                          int(N), int(K), int(group_size), int(quant_op), int(weight_bits),
+                          int(sa), int(sb), int(ss), int(sc), int(sd), _stream_ptr(stream))
     _lib.check(st, "device_gemv")
 
 
@@ -172,8 +191,9 @@ class GemvAdaptor:
             self.group_size, self.batch_count = int(group_size), int(batch_count)
             self.batch_strides = (batch_stride_A, batch_stride_B, batch_stride_scale, batch_stride_C, batch_stride_D)
 
-    def __init__(self, quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4):
-        self.quant_op, self.weight_bits = WeightOnlyQuantOp(quant_op), int(weight_bits)
+    def __init__(self, quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, element=None):
+        """element: "f16" / "bf16" (the reference's ElementB / ElementScale / ElementOutput), None = from ref_B."""
+        self.quant_op, self.weight_bits, self.element = WeightOnlyQuantOp(quant_op), int(weight_bits), element
         self._args = None
 
     def initialize(self, args, stream=None):
@@ -191,7 +211,7 @@ class GemvAdaptor:
         zero = a.ref_zero_point if self.quant_op == WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS else None
         device_gemv(a.ref_A, a.ref_B, a.ref_scale, zero, a.ref_C, a.ref_D, a.batch_count, m, n, k, a.group_size,
                     self.quant_op, self.weight_bits, stream,
-                    a.batch_strides if (a.batch_count != 1 or any(a.batch_strides)) else None)
+                    a.batch_strides if (a.batch_count != 1 or any(a.batch_strides)) else None, self.element)
 
     def __call__(self, args, stream=None):
         self.initialize(args, stream)
@@ -199,9 +219,11 @@ class GemvAdaptor:
 
 
 def dequantize(ptr_A, ptr_scale, ptr_zero_point, ptr_out, M, K, group_size,
-               quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, stream=None):
-    """Writes dequantised weights [M][K] fp16 with the kernels' own converter + dequantiser."""
-    st = _lib.lib().mgemv_dequantize(_dev_ptr(ptr_A), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_out),
+               quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, stream=None, element=None):
+    """Writes dequantised weights [M][K] (fp16, or bf16 with element="bf16" / a torch.bfloat16 scale
+    tensor) with the kernels' own converter + dequantiser."""
+    fn = _lib.lib().mgemv_dequantize_bf16 if _is_bf16(element, ptr_scale) else _lib.lib().mgemv_dequantize
+    st = fn(_dev_ptr(ptr_A), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_out),
                                      int(M), int(K), int(group_size), int(quant_op), int(weight_bits),
                                      _stream_ptr(stream))
     _lib.check(st, "dequantize")

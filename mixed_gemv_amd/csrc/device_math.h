@@ -171,6 +171,109 @@ __device__ __forceinline__ void dot2_row_bcast(float& acc, uint32_t x, half2_t d
 // Call this once after the last dot of a chain, before the accumulator is consumed.
 __device__ __forceinline__ void settle_dot_chain(float& acc) { asm volatile("s_nop 4" : "+v"(acc)); }
 
+// ---------------------------------------------------------------------------------------------
+// bfloat16 activations / scales / outputs.
+//
+// The reference's bf16 converters (gemv/interleaved_numeric_conversion.h:130-183 for int8,
+// :340-401 for int4) produce the exact integer q as a bf16, and its dequantiser
+// (gemv/warp/warp_dequantizer.h:52-59) multiplies by the scale and adds the zero term, each
+// rounded to bf16.  This target has no packed bf16 arithmetic, so both steps run in fp32, where
+// q * s is exact (at most 8 x 8 significant bits), and v_cvt_pk_bf16_f32 rounds to nearest even;
+// for the sum, rounding the fp32 sum to bf16 equals rounding the exact sum once (24 >= 2*8+2).
+// Values are kept as packed pairs of bf16 bit patterns, (low, high) = ascending k.
+//
+// Two forms, as for fp16.  With 8u (int4) or u (int8) from v_cvt_f32_ubyteN:
+//   fused    fma(8u, s/8, -8s) resp. fma(u, s, -128s): exact, hence = q*s, for 0 < s < 2^119
+//            (s/8 never underflows the fp32 subnormals, -8s / -128s stays finite; for s > 0 a zero
+//            product is +0 on both routes);
+//   general  (8u - 64) * (s/8) resp. (u - 128) * s: exact for every finite s, with the sign of
+//            a zero product as the reference's multiply gives it.
+// ---------------------------------------------------------------------------------------------
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kActF16 = 0;
+constexpr int kActBf16 = 1;
+
+__device__ __forceinline__ float bf16_low_to_f32(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
+__device__ __forceinline__ float bf16_high_to_f32(uint32_t bits) { return __builtin_bit_cast(float, bits & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2_t));
+}
+template <int BYTE>
+__device__ __forceinline__ float byte_to_f32(uint32_t v) {
+  return (float)((v >> (8 * BYTE)) & 0xffu);  // v_cvt_f32_ubyteN
+}
+
+// bf16 bit pattern of a scale for which the fused form is exact (both weight widths): 0x0001 .. 0x7aff.
+__device__ __forceinline__ bool fused_form_ok_bf16(uint32_t scale_bits) { return ((scale_bits & 0xffffu) - 1u) < 0x7affu; }
+
+struct Bf16Scale {
+  float mul;  // int4: s/8; int8: s
+  float add;  // fused form: -8s resp. -128s; general form: unused
+  float z;    // additive zero
+};
+
+template <int BITS, bool FUSED>
+__device__ __forceinline__ Bf16Scale make_bf16_scale(uint32_t s_bits, uint32_t z_bits) {
+  const float s = bf16_low_to_f32(s_bits);
+  Bf16Scale f;
+  f.mul = BITS == 4 ? s * 0.125f : s;
+  f.add = FUSED ? s * (BITS == 4 ? -8.0f : -128.0f) : 0.0f;
+  f.z = bf16_low_to_f32(z_bits);
+  return f;
+}
+
+// (a, b): the integers 8u (int4) or u (int8) of a k-adjacent pair -> packed bf16 pair of
+// rn(rn(q s) + z) resp. rn(q s).
+template <int BITS, bool HAS_ZERO, bool FUSED>
+__device__ __forceinline__ uint32_t dequant_pair_bf16(float a, float b, const Bf16Scale& f) {
+  float p0, p1;
+  if constexpr (FUSED) {
+    p0 = __builtin_fmaf(a, f.mul, f.add);
+    p1 = __builtin_fmaf(b, f.mul, f.add);
+  } else {
+    constexpr float kBias = BITS == 4 ? 64.0f : 128.0f;
+    p0 = (a - kBias) * f.mul;
+    p1 = (b - kBias) * f.mul;
+  }
+  uint32_t d = pack_bf16(p0, p1);
+  if constexpr (HAS_ZERO) d = pack_bf16(bf16_low_to_f32(d) + f.z, bf16_high_to_f32(d) + f.z);
+  return d;
+}
+
+// int4: the fields of elements (2,3) sit at bits 3-6 of bytes 0 and 2, those of (6,7) at bits 3-6
+// of bytes 1 and 3; (0,1) and (4,5) come to bytes 0 and 2 after a shift by 4 resp. a rotation
+// by 12 (tile_layout.h).  A masked byte converts to 8u.
+template <bool HAS_ZERO, bool FUSED>
+__device__ __forceinline__ void dequant_int4_word_bf16(uint32_t w, const ConvertRegs& c, const Bf16Scale& f,
+                                                       uint32_t (&d)[4]) {
+  const uint32_t e01 = (w >> 4) & c.mask3;
+  const uint32_t e23 = w & c.mask3;
+  const uint32_t e45 = __builtin_amdgcn_alignbit(w, w, 12) & c.mask3;
+  const uint32_t e67 = w & 0x78007800u;
+  d[0] = dequant_pair_bf16<4, HAS_ZERO, FUSED>(byte_to_f32<0>(e01), byte_to_f32<2>(e01), f);
+  d[1] = dequant_pair_bf16<4, HAS_ZERO, FUSED>(byte_to_f32<0>(e23), byte_to_f32<2>(e23), f);
+  d[2] = dequant_pair_bf16<4, HAS_ZERO, FUSED>(byte_to_f32<0>(e45), byte_to_f32<2>(e45), f);
+  d[3] = dequant_pair_bf16<4, HAS_ZERO, FUSED>(byte_to_f32<1>(e67), byte_to_f32<3>(e67), f);
+}
+
+// int8: 4 biased bytes in natural order.
+template <bool HAS_ZERO, bool FUSED>
+__device__ __forceinline__ void dequant_int8_word_bf16(uint32_t w, const Bf16Scale& f, uint32_t (&d)[2]) {
+  d[0] = dequant_pair_bf16<8, HAS_ZERO, FUSED>(byte_to_f32<0>(w), byte_to_f32<1>(w), f);
+  d[1] = dequant_pair_bf16<8, HAS_ZERO, FUSED>(byte_to_f32<2>(w), byte_to_f32<3>(w), f);
+}
+
+// bf16 counterpart of dot2_row_bcast (same hazards, same settle_dot_chain afterwards).
+template <int SRC>
+__device__ __forceinline__ void dot2_row_bcast_bf16(float& acc, uint32_t x, uint32_t d) {
+  static_assert(SRC >= 0 && SRC < 16, "source lane within a 16-lane DPP row");
+  asm("v_dot2c_f32_bf16_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+      : "+v"(acc)
+      : "v"(x), "v"(d), "n"(SRC));
+}
+
 // Raw buffer descriptor: base pointer + byte count; out-of-range lanes read zero.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);

@@ -279,30 +279,54 @@ __device__ __forceinline__ void compute_word(float (&acc)[MB], uint32_t w, const
   }
 }
 
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT, int I>
+// The same for bf16 operands; SHORT selects the fused form.
+template <int BITS, bool HAS_ZERO, bool SHORT, int MB, int I, int J>
+__device__ __forceinline__ void compute_word_bf16(float (&acc)[MB], uint32_t w,
+                                                  const uint32_t (&x)[MB][BITS == 4 ? 4 : 2], const ConvertRegs& c,
+                                                  const Bf16Scale& f) {
+  constexpr int kPairs = BITS == 4 ? 4 : 2;
+  uint32_t d[kPairs];
+  if constexpr (BITS == 4) dequant_int4_word_bf16<HAS_ZERO, SHORT>(w, c, f, d);
+  else dequant_int8_word_bf16<HAS_ZERO, SHORT>(w, f, d);
+#pragma unroll
+  for (int h = 0; h < kPairs; ++h) {
+#pragma unroll
+    for (int m = 0; m < MB; ++m) dot2_row_bcast_bf16<4 * I + J>(acc[m], x[m][h], d[h]);
+  }
+}
+
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT, int I, int ACT>
 __device__ __forceinline__ void compute_block(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
                                               const ConvertRegs& c) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
   constexpr int gi = I * GROUPS_PER_RUN / kBlocksPerUnit;
-  const half2_t s2 = splat_low(f.s[gi]);
-  half2_t z2 = half2_t{};
-  if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
-  ShortFormScale sf{};
-  if constexpr (BITS == 4 && SHORT) sf = make_short_form_scale(s2);
-  compute_word<BITS, kHasZero, SHORT, MB, I, 0>(acc, f.w[I][0], f.x, c, s2, z2, sf);
-  compute_word<BITS, kHasZero, SHORT, MB, I, 1>(acc, f.w[I][1], f.x, c, s2, z2, sf);
-  compute_word<BITS, kHasZero, SHORT, MB, I, 2>(acc, f.w[I][2], f.x, c, s2, z2, sf);
-  compute_word<BITS, kHasZero, SHORT, MB, I, 3>(acc, f.w[I][3], f.x, c, s2, z2, sf);
+  if constexpr (ACT == kActBf16) {
+    const Bf16Scale bs = make_bf16_scale<BITS, SHORT>(f.s[gi], kHasZero ? f.z[gi] : 0u);
+    compute_word_bf16<BITS, kHasZero, SHORT, MB, I, 0>(acc, f.w[I][0], f.x, c, bs);
+    compute_word_bf16<BITS, kHasZero, SHORT, MB, I, 1>(acc, f.w[I][1], f.x, c, bs);
+    compute_word_bf16<BITS, kHasZero, SHORT, MB, I, 2>(acc, f.w[I][2], f.x, c, bs);
+    compute_word_bf16<BITS, kHasZero, SHORT, MB, I, 3>(acc, f.w[I][3], f.x, c, bs);
+  } else {
+    const half2_t s2 = splat_low(f.s[gi]);
+    half2_t z2 = half2_t{};
+    if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
+    ShortFormScale sf{};
+    if constexpr (BITS == 4 && SHORT) sf = make_short_form_scale(s2);
+    compute_word<BITS, kHasZero, SHORT, MB, I, 0>(acc, f.w[I][0], f.x, c, s2, z2, sf);
+    compute_word<BITS, kHasZero, SHORT, MB, I, 1>(acc, f.w[I][1], f.x, c, s2, z2, sf);
+    compute_word<BITS, kHasZero, SHORT, MB, I, 2>(acc, f.w[I][2], f.x, c, s2, z2, sf);
+    compute_word<BITS, kHasZero, SHORT, MB, I, 3>(acc, f.w[I][3], f.x, c, s2, z2, sf);
+  }
 }
 
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT>
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool SHORT, int ACT>
 __device__ __forceinline__ void compute_unit_form(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
                                                   const ConvertRegs& regs) {
-  const ConvertRegs c = (BITS == 4 && !SHORT) ? general_form_regs(regs) : regs;
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 0>(acc, f, c);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 1>(acc, f, c);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 2>(acc, f, c);
-  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 3>(acc, f, c);
+  const ConvertRegs c = (ACT == kActF16 && BITS == 4 && !SHORT) ? general_form_regs(regs) : regs;
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 0, ACT>(acc, f, c);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 1, ACT>(acc, f, c);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 2, ACT>(acc, f, c);
+  compute_block<BITS, QOP, MB, GROUPS_PER_RUN, SHORT, 3, ACT>(acc, f, c);
   // The two forms meet again after this call, and the compiler may place a register copy of
   // the accumulators at that join: make them safe to read by any instruction first.
 #pragma unroll
@@ -310,26 +334,28 @@ __device__ __forceinline__ void compute_unit_form(float (&acc)[MB], const UnitFr
 }
 
 // True when the scale of every lane of the wave (all groups of the unit) permits the short
-// int4 dequantiser; wave-uniform, so the choice costs one scalar branch per unit.
-template <typename Bits, int GROUPS_PER_RUN>
+// (fp16, int4) resp. fused (bf16) dequantiser; wave-uniform, so the choice costs one scalar
+// branch per unit.
+template <int ACT, typename Bits, int GROUPS_PER_RUN>
 __device__ __forceinline__ bool wave_scales_permit_short_form(const Bits (&scale_bits)[GROUPS_PER_RUN]) {
   bool ok = true;
 #pragma unroll
-  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) ok = ok && short_form_ok(scale_bits[gi]);
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi)
+    ok = ok && (ACT == kActBf16 ? fused_form_ok_bf16(scale_bits[gi]) : short_form_ok(scale_bits[gi]));
   return __builtin_amdgcn_ballot_w64(!ok) == 0;
 }
 
 // short_allowed: wave-uniform.
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN>
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, int ACT = kActF16>
 __device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
                                              const ConvertRegs& c, bool short_allowed) {
-  if constexpr (BITS == 4) {
-    if (short_allowed && wave_scales_permit_short_form(f.s)) {
-      compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, true>(acc, f, c);
+  if constexpr (BITS == 4 || ACT == kActBf16) {
+    if (short_allowed && wave_scales_permit_short_form<ACT>(f.s)) {
+      compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, true, ACT>(acc, f, c);
       return;
     }
   }
-  compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, false>(acc, f, c);
+  compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, false, ACT>(acc, f, c);
 }
 
 // Sum over the four k slices of a wave: lanes l, l+16, l+32, l+48 hold the same row.
@@ -342,12 +368,19 @@ __device__ __forceinline__ float reduce_k_slices(float v) {
 
 // Epilogue: fp32 add of the bias, one rounding to fp16
 // (host/mixed_gemv.h:102-103; epilogue/threadblock/epilogue.h:50-75).
+template <int ACT>
 __device__ __forceinline__ void store_outputs(const GemvTail& tail, bool has_bias, int n_out, int m, int tile, int lane,
                                               float sum) {
   const int n = tile * kTileRows + lane;
   if (lane < kTileRows && n < n_out) {
-    if (has_bias) sum += (float)tail.bias[n];
-    tail.y[(size_t)m * (size_t)n_out + n] = (half_t)sum;
+    if constexpr (ACT == kActBf16) {
+      const uint16_t* bias = reinterpret_cast<const uint16_t*>(tail.bias);
+      if (has_bias) sum += bf16_low_to_f32(bias[n]);
+      reinterpret_cast<uint16_t*>(tail.y)[(size_t)m * (size_t)n_out + n] = (uint16_t)pack_bf16(sum, 0.0f);
+    } else {
+      if (has_bias) sum += (float)tail.bias[n];
+      tail.y[(size_t)m * (size_t)n_out + n] = (half_t)sum;
+    }
   }
 }
 
@@ -375,9 +408,11 @@ __device__ __forceinline__ void finish_tile(float (&acc)[MB], float* slot) {
 // split_k * MB * 64 floats.
 // One activation row, one group per run: ask for 6 resident waves per SIMD (at most 80 VGPRs).
 // The allocation unit is 8 registers, so 81 would already cost a whole wave of occupancy.
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI>
-__global__ void __launch_bounds__(kWave * (MB >= 3 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
-__attribute__((amdgpu_waves_per_eu(MB == 1 && GROUPS_PER_RUN == 1 ? 6 : 1)))
+// ACT: kActF16 or kActBf16 -- the type of activations, scales, zeros, bias and outputs (the
+// pointers are typed as 16-bit storage either way).
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI, int ACT>
+__global__ void __launch_bounds__(kWave * (MB >= 3 || ACT == kActBf16 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
+__attribute__((amdgpu_waves_per_eu(ACT == kActF16 && MB == 1 && GROUPS_PER_RUN == 1 ? 6 : 1)))
 gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
                 uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
   extern __shared__ float partials[];
@@ -464,7 +499,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
     const ConvertRegs c = make_convert_regs();
     if (total == 1) {
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, short_ok);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
       if constexpr (MULTI) finish_tile<MB>(acc, slot);
     } else {
       // The prefetches are unconditional: past the wave's last unit every weight offset is out
@@ -475,7 +510,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         advance<MULTI>(cur, walk);
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
         __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
-        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fa, c, short_ok);
+        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
         if constexpr (MULTI) {
           if (--pending == 0) {
             finish_tile<MB>(acc, slot);
@@ -487,7 +522,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
         __builtin_amdgcn_sched_barrier(0);
         if (u + 1 < total) {
-          compute_unit<BITS, QOP, MB, GROUPS_PER_RUN>(acc, fb, c, short_ok);
+          compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fb, c, short_ok);
           if constexpr (MULTI) {
             if (--pending == 0) {
               finish_tile<MB>(acc, slot);
@@ -520,7 +555,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       sum = (((sum + a0) + a1) + a2) + a3;
     }
     for (; w < split_k; ++w) sum += part[w * MB * kWave];
-    store_outputs(tail, has_bias, p.n_out, m, tile_begin + j, lane_c, reduce_k_slices(sum));
+    store_outputs<ACT>(tail, has_bias, p.n_out, m, tile_begin + j, lane_c, reduce_k_slices(sum));
   }
 }
 
@@ -661,7 +696,7 @@ __device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<
                                                   half2_t col_scale2, bool short_allowed) {
   if constexpr (BITS == 4) {
     bool take_short = short_allowed;
-    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form(f.s);
+    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form<kActF16>(f.s);
     if (take_short) {
       compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, true>(acc, f, xa, c, col_scale2);
       return;
@@ -743,7 +778,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
       if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
         col_scale[t] = splat(p.scale[row[t]]);
         const uint32_t bits[1] = {as_u32(col_scale[t])};
-        short_ok[t] = short_ok[t] && wave_scales_permit_short_form(bits);
+        short_ok[t] = short_ok[t] && wave_scales_permit_short_form<kActF16>(bits);
       }
     }
     const ConvertRegs c = make_convert_regs();
@@ -965,7 +1000,7 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
   if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
     col_scale = splat(p.scale[row]);
     const uint32_t bits[1] = {as_u32(col_scale)};
-    short_ok = short_ok && wave_scales_permit_short_form(bits);
+    short_ok = short_ok && wave_scales_permit_short_form<kActF16>(bits);
   }
   const ConvertRegs c = make_convert_regs();
 
@@ -1039,7 +1074,7 @@ struct DequantParams {
 
 // One wave per unit; writes the dequantised weights of its 16 rows x kStepK columns with the
 // same converters, and the same wave-uniform choice between them, as the GEMV kernels.
-template <int BITS, int QOP>
+template <int BITS, int QOP, int ACT>
 __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, half_t* __restrict__ out) {
   using G = Geometry<BITS>;
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
@@ -1069,8 +1104,8 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, 
     }
     s_bits[i] = (uint32_t)__builtin_bit_cast(uint16_t, s[i]);
   }
-  const bool take_short =
-      BITS == 4 && (p.flags & kExactIntegerFormOnly) == 0 && wave_scales_permit_short_form(s_bits);
+  const bool take_short = (BITS == 4 || ACT == kActBf16) && (p.flags & kExactIntegerFormOnly) == 0 &&
+                          wave_scales_permit_short_form<ACT>(s_bits);
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i) {
     const int k0 = k_run + i * G::kChunkK;
@@ -1078,6 +1113,26 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, 
     const half2_t s2 = splat(s[i]), z2 = splat(z[i]);
     if (row >= p.n_out || k0 >= p.k) continue;
     half_t* dst = out + (size_t)row * (size_t)p.k + k0;
+    if constexpr (ACT == kActBf16) {
+      constexpr int kPairs = BITS == 4 ? 4 : 2;
+      const uint32_t z_bits = (uint32_t)__builtin_bit_cast(uint16_t, z[i]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t d[kPairs];
+        if (take_short) {
+          const Bf16Scale bs = make_bf16_scale<BITS, true>(s_bits[i], z_bits);
+          if constexpr (BITS == 4) dequant_int4_word_bf16<kHasZero, true>(w[j], c, bs, d);
+          else dequant_int8_word_bf16<kHasZero, true>(w[j], bs, d);
+        } else {
+          const Bf16Scale bs = make_bf16_scale<BITS, false>(s_bits[i], z_bits);
+          if constexpr (BITS == 4) dequant_int4_word_bf16<kHasZero, false>(w[j], c, bs, d);
+          else dequant_int8_word_bf16<kHasZero, false>(w[j], bs, d);
+        }
+#pragma unroll
+        for (int h = 0; h < kPairs; ++h) *reinterpret_cast<uint32_t*>(dst + j * 2 * kPairs + h * 2) = d[h];
+      }
+      continue;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if constexpr (BITS == 4) {
@@ -1120,6 +1175,7 @@ struct PlanKnobs {
   int split_k = 0, tiles_per_wg = 0, tiles_per_wave = 0, workgroups = 0;
   int matrix_core_min_batch = 0;
   int matrix_core_variant = MGEMV_MATRIX_CORE_AUTO;
+  bool wide_waves = false;  // the kernel is one of those compiled for at most 8 waves per workgroup
 };
 
 // Tuned plans by problem: (n_out, k, weight bits, group size or 0 for any, m_batch) -> knobs.
@@ -1216,7 +1272,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   //    launch stays under ~8k waves, and fall back to two units per wave when that still
   //    leaves >= 4096 waves (8192x8192: 10.6 us at 8 waves vs 11.2 us at 16).
   const int max_waves = mc ? kMaxWavesPerMfmaWorkgroup
-                        : m_batch >= 3            ? kMaxWavesPerWideWorkgroup
+                        : m_batch >= 3 || knobs.wide_waves ? kMaxWavesPerWideWorkgroup
                                                   : kMaxWavesPerWorkgroup;
   int split_k;
   if (groups <= 384) {
@@ -1340,55 +1396,61 @@ struct GemvLaunch {
   hipStream_t stream;
 };
 
-template <int BITS, int QOP, int MB, int GPR, bool MULTI>
+template <int BITS, int QOP, int MB, int GPR, bool MULTI, int ACT>
 hipError_t launch_gemv_kernel_m(const GemvLaunch& g) {
-  return launch(gemv_dpp_kernel<BITS, QOP, MB, GPR, MULTI>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
+  return launch(gemv_dpp_kernel<BITS, QOP, MB, GPR, MULTI, ACT>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
                 g.zero_add, g.n_out, g.k, pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups,
                 g.tail.num_groups, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
 }
 
-template <int BITS, int QOP, int MB, int GPR>
+template <int BITS, int QOP, int MB, int GPR, int ACT>
 hipError_t launch_gemv_kernel(const GemvLaunch& g) {
-  return g.plan.tiles_in_sequence > 1 ? launch_gemv_kernel_m<BITS, QOP, MB, GPR, true>(g)
-                                      : launch_gemv_kernel_m<BITS, QOP, MB, GPR, false>(g);
+  return g.plan.tiles_in_sequence > 1 ? launch_gemv_kernel_m<BITS, QOP, MB, GPR, true, ACT>(g)
+                                      : launch_gemv_kernel_m<BITS, QOP, MB, GPR, false, ACT>(g);
 }
 
-template <int BITS, int QOP, int MB>
+template <int BITS, int QOP, int MB, int ACT>
 hipError_t launch_gemv_gpr(const GemvLaunch& g, int gpr) {
   if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
-    return launch_gemv_kernel<BITS, QOP, MB, 1>(g);
+    return launch_gemv_kernel<BITS, QOP, MB, 1, ACT>(g);
   } else {
     switch (gpr) {
-      case 1: return launch_gemv_kernel<BITS, QOP, MB, 1>(g);
-      case 2: return launch_gemv_kernel<BITS, QOP, MB, 2>(g);
-      default: return launch_gemv_kernel<BITS, QOP, MB, 4>(g);
+      case 1: return launch_gemv_kernel<BITS, QOP, MB, 1, ACT>(g);
+      case 2: return launch_gemv_kernel<BITS, QOP, MB, 2, ACT>(g);
+      default: return launch_gemv_kernel<BITS, QOP, MB, 4, ACT>(g);
     }
   }
 }
 
-template <int BITS, int QOP>
+template <int BITS, int QOP, int ACT>
 hipError_t launch_gemv_mb(const GemvLaunch& g, int mb, int gpr) {
   switch (mb) {
-    case 1: return launch_gemv_gpr<BITS, QOP, 1>(g, gpr);
-    case 2: return launch_gemv_gpr<BITS, QOP, 2>(g, gpr);
-    case 3: return launch_gemv_gpr<BITS, QOP, 3>(g, gpr);
-    default: return launch_gemv_gpr<BITS, QOP, 4>(g, gpr);
+    case 1: return launch_gemv_gpr<BITS, QOP, 1, ACT>(g, gpr);
+    case 2: return launch_gemv_gpr<BITS, QOP, 2, ACT>(g, gpr);
+    case 3: return launch_gemv_gpr<BITS, QOP, 3, ACT>(g, gpr);
+    default: return launch_gemv_gpr<BITS, QOP, 4, ACT>(g, gpr);
   }
 }
 
-hipError_t launch_gemv(const GemvLaunch& g, int bits, int qop, int mb, int gpr) {
+template <int ACT>
+hipError_t launch_gemv_act(const GemvLaunch& g, int bits, int qop, int mb, int gpr) {
   if (bits == 4) {
     switch (qop) {
-      case 1: return launch_gemv_mb<4, 1>(g, mb, gpr);
-      case 2: return launch_gemv_mb<4, 2>(g, mb, gpr);
-      default: return launch_gemv_mb<4, 3>(g, mb, gpr);
+      case 1: return launch_gemv_mb<4, 1, ACT>(g, mb, gpr);
+      case 2: return launch_gemv_mb<4, 2, ACT>(g, mb, gpr);
+      default: return launch_gemv_mb<4, 3, ACT>(g, mb, gpr);
     }
   }
   switch (qop) {
-    case 1: return launch_gemv_mb<8, 1>(g, mb, gpr);
-    case 2: return launch_gemv_mb<8, 2>(g, mb, gpr);
-    default: return launch_gemv_mb<8, 3>(g, mb, gpr);
+    case 1: return launch_gemv_mb<8, 1, ACT>(g, mb, gpr);
+    case 2: return launch_gemv_mb<8, 2, ACT>(g, mb, gpr);
+    default: return launch_gemv_mb<8, 3, ACT>(g, mb, gpr);
   }
+}
+
+hipError_t launch_gemv(const GemvLaunch& g, int bits, int qop, int mb, int gpr, int act) {
+  return act == kActBf16 ? launch_gemv_act<kActBf16>(g, bits, qop, mb, gpr)
+                         : launch_gemv_act<kActF16>(g, bits, qop, mb, gpr);
 }
 
 template <int BITS, int QOP, int GPR, int T>
@@ -1482,26 +1544,22 @@ hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int 
   }
 }
 
-template <int BITS>
+template <int BITS, int ACT>
 hipError_t launch_dequant(const DequantParams& p, int qop, half_t* out, hipStream_t stream) {
   const long long units = (long long)p.tiles * p.ksteps;
   const dim3 block(256), grid((unsigned)((units + 3) / 4));
   switch (qop) {
-    case 1: return launch(dequantize_kernel<BITS, 1>, grid, block, 0, stream, p, out);
-    case 2: return launch(dequantize_kernel<BITS, 2>, grid, block, 0, stream, p, out);
-    default: return launch(dequantize_kernel<BITS, 3>, grid, block, 0, stream, p, out);
+    case 1: return launch(dequantize_kernel<BITS, 1, ACT>, grid, block, 0, stream, p, out);
+    case 2: return launch(dequantize_kernel<BITS, 2, ACT>, grid, block, 0, stream, p, out);
+    default: return launch(dequantize_kernel<BITS, 3, ACT>, grid, block, 0, stream, p, out);
   }
 }
 
-}  // namespace mgemv
-
-extern "C" {
-
-int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
-                       const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k,
-                       int group_size, int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x,
-                       int64_t stride_scale, int64_t stride_bias, int64_t stride_y, void* stream) {
-  using namespace mgemv;
+// act: kActF16 or kActBf16, the type behind every 16-bit operand.
+int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+             const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k, int group_size,
+             int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
+             int64_t stride_bias, int64_t stride_y, void* stream, int act) {
   if (batch_count < 1 || batch_count > 65535) return MGEMV_ERR_BATCH;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
@@ -1518,7 +1576,12 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
   g.n_out = n_out;
   g.k = k;
   g.group_size = group_size;
-  g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs_for(n_out, k, weight_bits, group_size, m_batch));
+  PlanKnobs knobs = knobs_for(n_out, k, weight_bits, group_size, m_batch);
+  if (act == kActBf16) {
+    knobs.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1;  // bf16: VALU kernel only, ...
+    knobs.wide_waves = true;                              // ... whose fp32 dequantiser wants the registers of 8-wave workgroups
+  }
+  g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs);
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
@@ -1560,21 +1623,13 @@ int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* s
     g.x = reinterpret_cast<const half_t*>(x) + (size_t)m0 * (size_t)k;
     g.tail.y = reinterpret_cast<half_t*>(y) + (size_t)m0 * (size_t)n_out;
     g.lds = (size_t)g.plan.tiles_in_sequence * g.plan.tiles_per_wg * g.plan.split_k * mb * kWave * sizeof(float);
-    if (launch_gemv(g, weight_bits, quant_op, mb, gpr) != hipSuccess) return MGEMV_ERR_LAUNCH;
+    if (launch_gemv(g, weight_bits, quant_op, mb, gpr, act) != hipSuccess) return MGEMV_ERR_LAUNCH;
   }
   return MGEMV_OK;
 }
 
-int mgemv_gemv(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
-               const uint16_t* bias, uint16_t* y, int n_out, int m_batch, int k, int group_size, int quant_op,
-               int weight_bits, void* stream) {
-  return mgemv_gemv_batched(weights, x, scale, zero_add, bias, y, 1, n_out, m_batch, k, group_size, quant_op,
-                            weight_bits, 0, 0, 0, 0, 0, stream);
-}
-
-int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t* zero_add, uint16_t* out, int n_out,
-                     int k, int group_size, int quant_op, int weight_bits, void* stream) {
-  using namespace mgemv;
+int dequantize_any(const void* weights, const uint16_t* scale, const uint16_t* zero_add, uint16_t* out, int n_out,
+                   int k, int group_size, int quant_op, int weight_bits, void* stream, int act) {
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(out) % 4) return MGEMV_ERR_ALIGNMENT;
@@ -1588,10 +1643,62 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
   p.tiles = num_tiles(n_out);
   p.ksteps = num_ksteps(k, weight_bits);
   p.flags = g_dequant_flags.load();
-  const hipError_t e = weight_bits == 4
-                           ? launch_dequant<4>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream))
-                           : launch_dequant<8>(p, quant_op, reinterpret_cast<half_t*>(out), static_cast<hipStream_t>(stream));
+  half_t* const o = reinterpret_cast<half_t*>(out);
+  hipStream_t const st = static_cast<hipStream_t>(stream);
+  hipError_t e;
+  if (act == kActBf16)
+    e = weight_bits == 4 ? launch_dequant<4, kActBf16>(p, quant_op, o, st) : launch_dequant<8, kActBf16>(p, quant_op, o, st);
+  else
+    e = weight_bits == 4 ? launch_dequant<4, kActF16>(p, quant_op, o, st) : launch_dequant<8, kActF16>(p, quant_op, o, st);
   return e == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+}
+
+}  // namespace mgemv
+
+extern "C" {
+
+int mgemv_gemv_batched(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+                       const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k,
+                       int group_size, int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x,
+                       int64_t stride_scale, int64_t stride_bias, int64_t stride_y, void* stream) {
+  return mgemv::gemv_any(weights, x, scale, zero_add, bias, y, batch_count, n_out, m_batch, k, group_size, quant_op,
+                         weight_bits, stride_weights, stride_x, stride_scale, stride_bias, stride_y, stream,
+                         mgemv::kActF16);
+}
+
+int mgemv_gemv_batched_bf16(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+                            const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k,
+                            int group_size, int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x,
+                            int64_t stride_scale, int64_t stride_bias, int64_t stride_y, void* stream) {
+  return mgemv::gemv_any(weights, x, scale, zero_add, bias, y, batch_count, n_out, m_batch, k, group_size, quant_op,
+                         weight_bits, stride_weights, stride_x, stride_scale, stride_bias, stride_y, stream,
+                         mgemv::kActBf16);
+}
+
+int mgemv_gemv_bf16(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+                    const uint16_t* bias, uint16_t* y, int n_out, int m_batch, int k, int group_size, int quant_op,
+                    int weight_bits, void* stream) {
+  return mgemv_gemv_batched_bf16(weights, x, scale, zero_add, bias, y, 1, n_out, m_batch, k, group_size, quant_op,
+                                 weight_bits, 0, 0, 0, 0, 0, stream);
+}
+
+int mgemv_dequantize_bf16(const void* weights, const uint16_t* scale, const uint16_t* zero_add, uint16_t* out, int n_out,
+                          int k, int group_size, int quant_op, int weight_bits, void* stream) {
+  return mgemv::dequantize_any(weights, scale, zero_add, out, n_out, k, group_size, quant_op, weight_bits, stream,
+                               mgemv::kActBf16);
+}
+
+int mgemv_gemv(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+               const uint16_t* bias, uint16_t* y, int n_out, int m_batch, int k, int group_size, int quant_op,
+               int weight_bits, void* stream) {
+  return mgemv_gemv_batched(weights, x, scale, zero_add, bias, y, 1, n_out, m_batch, k, group_size, quant_op,
+                            weight_bits, 0, 0, 0, 0, 0, stream);
+}
+
+int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t* zero_add, uint16_t* out, int n_out,
+                     int k, int group_size, int quant_op, int weight_bits, void* stream) {
+  return mgemv::dequantize_any(weights, scale, zero_add, out, n_out, k, group_size, quant_op, weight_bits, stream,
+                               mgemv::kActF16);
 }
 
 int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave, int max_workgroups) {

@@ -180,6 +180,27 @@ int mgemv_fold_zero_points(uint16_t* out, const uint16_t* scales, const int8_t* 
   return MGEMV_OK;
 }
 
+int mgemv_fold_zero_points_bf16(uint16_t* out, const uint16_t* scales, const int8_t* zeros, size_t n) {
+  if (n == 0) return MGEMV_OK;
+  if (out == nullptr || scales == nullptr || zeros == nullptr) return MGEMV_ERR_NULL_POINTER;
+  for (size_t i = 0; i < n; ++i) {
+    // -z has at most 8 significant bits: exact in bfloat16.  The binary32 product of two
+    // bfloat16 values is exact, so one rounding (nearest even) is the correctly rounded multiply.
+    const uint32_t s_bits = (uint32_t)scales[i] << 16;
+    float s;
+    std::memcpy(&s, &s_bits, 4);
+    const float prod = (float)(-(int)zeros[i]) * s;
+    uint32_t bits;
+    std::memcpy(&bits, &prod, 4);
+    if ((bits & 0x7fffffffu) > 0x7f800000u) {
+      out[i] = (uint16_t)((bits >> 16) | 0x0040u);  // NaN stays NaN
+    } else {
+      out[i] = (uint16_t)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+    }
+  }
+  return MGEMV_OK;
+}
+
 size_t mgemv_preprocessed_size(const size_t* shape, int rank, int quant_type) {
   size_t experts, k, n_out;
   const int bits = bits_of_quant_type(quant_type);

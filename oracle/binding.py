@@ -50,6 +50,21 @@ def lib():
         h.orc_dequantize.argtypes = [vp, vp, vp, vp] + [c.c_int] * 6
         h.orc_gemv.restype = c.c_int
         h.orc_gemv.argtypes = [vp, vp, vp, vp, vp, vp] + [c.c_int] * 8
+        h.orc_dequantize_bf16.restype = c.c_int
+        h.orc_dequantize_bf16.argtypes = h.orc_dequantize.argtypes
+        h.orc_gemv_bf16.restype = c.c_int
+        h.orc_gemv_bf16.argtypes = h.orc_gemv.argtypes
+        h.orc_fold_zero_points_bf16.argtypes = [vp, vp, vp, c.c_size_t]
+        h.orc_bf16_to_f32.restype = c.c_float
+        h.orc_bf16_to_f32.argtypes = [c.c_uint16]
+        h.orc_f32_to_bf16.restype = c.c_uint16
+        h.orc_f32_to_bf16.argtypes = [c.c_float]
+        for name in ("orc_bf16_mul", "orc_bf16_add"):
+            getattr(h, name).restype = c.c_uint16
+            getattr(h, name).argtypes = [c.c_uint16, c.c_uint16]
+        for name, nargs in (("orc_bf16_to_f32_n", 2), ("orc_f32_to_bf16_n", 2), ("orc_bf16_mul_n", 3),
+                            ("orc_bf16_add_n", 3)):
+            getattr(h, name).argtypes = [vp] * nargs + [c.c_size_t]
         h.orc_max_threads.restype = c.c_int
         h.orc_fill_int8.argtypes = [vp, c.c_size_t, c.c_uint64, c.c_int, c.c_int]
         h.orc_fill_uniform_f16.argtypes = [vp, c.c_size_t, c.c_uint64, c.c_float, c.c_float]
@@ -130,6 +145,63 @@ def h_fma_array(a, b, c):
     out = np.empty(a.shape, dtype=np.uint16)
     lib().orc_h_fma_n(_p(out), _p(a), _p(b), _p(c), a.size)
     return out
+
+
+# ---- bfloat16 (bit patterns travel as uint16 arrays; numpy has no such dtype) --------------
+
+def bf16_to_f32_array(bits):
+    b = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(b.shape, dtype=np.float32)
+    lib().orc_bf16_to_f32_n(_p(out), _p(b), b.size)
+    return out
+
+
+def f32_to_bf16_array(values):
+    v = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(v.shape, dtype=np.uint16)
+    lib().orc_f32_to_bf16_n(_p(out), _p(v), v.size)
+    return out
+
+
+def bf16_mul_array(a, b):
+    return _binary(lib().orc_bf16_mul_n, a, b)
+
+
+def bf16_add_array(a, b):
+    return _binary(lib().orc_bf16_add_n, a, b)
+
+
+def fold_zero_points_bf16(scales, zeros):
+    s = np.ascontiguousarray(scales, dtype=np.uint16)
+    z = np.ascontiguousarray(zeros, dtype=np.int8)
+    out = np.empty(s.shape, dtype=np.uint16)
+    lib().orc_fold_zero_points_bf16(_p(out), _p(s), _p(z), s.size)
+    return out
+
+
+def dequantize_bf16(W, scale, zero, n_out, k, group_size, quant_op, bits):
+    """As dequantize, with bf16 bit patterns (uint16) for scale / folded zero / result."""
+    W = np.ascontiguousarray(W)
+    s = np.ascontiguousarray(scale, dtype=np.uint16)
+    z, zk = _zero_args(zero, quant_op)
+    out = np.empty((n_out, k), dtype=np.uint16)
+    rc = lib().orc_dequantize_bf16(_p(out), _p(W), _p(s), _p(z), zk, n_out, k, group_size, quant_op, bits)
+    assert rc == 0
+    return out
+
+
+def gemv_bf16(W, x, scale, zero, bias, n_out, m_batch, k, group_size, quant_op, bits, threads=1):
+    """HOST_CHECK GEMV with bfloat16 elements; every 16-bit operand and the result are uint16 bit patterns."""
+    W = np.ascontiguousarray(W)
+    xx = np.ascontiguousarray(x, dtype=np.uint16)
+    s = np.ascontiguousarray(scale, dtype=np.uint16)
+    z, zk = _zero_args(zero, quant_op)
+    b = np.ascontiguousarray(bias, dtype=np.uint16) if bias is not None else None
+    y = np.empty((m_batch, n_out), dtype=np.uint16)
+    rc = lib().orc_gemv_bf16(_p(y), _p(W), _p(xx), _p(s), _p(z), _p(b), zk, n_out, m_batch, k, group_size, quant_op,
+                             bits, threads)
+    assert rc == 0
+    return y
 
 
 # ---- host utilities ----------------------------------------------------------------------

@@ -27,6 +27,15 @@
  *   orc_gemv                           numpy restatement, one-hot / all-ones closed forms,
  *                                      float64 bound
  *   orc_fill_*                         definitional (they are the generator); statistics only
+ *   orc_bf16_to_f32 / orc_f32_to_bf16  exhaustive / 4 M random floats against torch.bfloat16; ties
+ *   orc_bf16_mul / orc_bf16_add        exact rational arithmetic (fractions) on random and edge pairs
+ *   orc_dequantize_bf16 / orc_gemv_bf16 / orc_fold_zero_points_bf16
+ *                                      the same loops as the fp16 functions with the element
+ *                                      arithmetic swapped; torch.bfloat16 restatements, one-hot and
+ *                                      unit-weight closed forms.  The reference holds no bf16 test or
+ *                                      vector (its bf16 instantiation does not compile,
+ *                                      gemv/threadblock/default_dq_mma_simt.h:133-134), so these are
+ *                                      pinned by the mathematics alone.
  */
 #include <stddef.h>
 #include <stdint.h>
@@ -120,6 +129,41 @@ static inline uint16_t h_from_int(int v) { return orc_f32_to_f16((float)v); }
 
 ORC_API uint16_t orc_h_mul(uint16_t a, uint16_t b) { return h_mul(a, b); }
 ORC_API uint16_t orc_h_add(uint16_t a, uint16_t b) { return h_add(a, b); }
+
+/* bfloat16 = the upper 16 bits of a binary32; conversion from binary32 rounds to nearest even
+ * (cutlass::bfloat16_t's conversion, which the reference's element types would use).  A product
+ * of two bfloat16 values is exact in binary32 (16 significant bits) and for a sum the double
+ * rounding 24 -> 8 bits is innocuous (24 >= 2*8+2), so one binary32 operation followed by this
+ * rounding is the correctly rounded bfloat16 operation. */
+ORC_API float orc_bf16_to_f32(uint16_t b) {
+  uint32_t bits = (uint32_t)b << 16;
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+ORC_API uint16_t orc_f32_to_bf16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u); /* quiet NaN */
+  uint32_t kept = x >> 16, rem = x & 0xffffu;
+  if (rem > 0x8000u || (rem == 0x8000u && (kept & 1u))) kept += 1; /* carries into the exponent / to inf correctly */
+  return (uint16_t)kept;
+}
+static inline uint16_t b_mul(uint16_t a, uint16_t b) { return orc_f32_to_bf16(orc_bf16_to_f32(a) * orc_bf16_to_f32(b)); }
+static inline uint16_t b_add(uint16_t a, uint16_t b) { return orc_f32_to_bf16(orc_bf16_to_f32(a) + orc_bf16_to_f32(b)); }
+ORC_API uint16_t orc_bf16_mul(uint16_t a, uint16_t b) { return b_mul(a, b); }
+ORC_API uint16_t orc_bf16_add(uint16_t a, uint16_t b) { return b_add(a, b); }
+
+/* Element type of activations / scales / zeros / outputs: the reference's ElementB = ElementScale =
+ * ElementOutput template arguments (host/mixed_gemv.h:24-31). */
+enum { ORC_ELEM_F16 = 0, ORC_ELEM_BF16 = 1 };
+static inline uint16_t e_mul(int elem, uint16_t a, uint16_t b) { return elem == ORC_ELEM_BF16 ? b_mul(a, b) : h_mul(a, b); }
+static inline uint16_t e_add(int elem, uint16_t a, uint16_t b) { return elem == ORC_ELEM_BF16 ? b_add(a, b) : h_add(a, b); }
+static inline uint16_t e_from_int(int elem, int v) { /* |v| <= 128: exact in either type */
+  return elem == ORC_ELEM_BF16 ? orc_f32_to_bf16((float)v) : orc_f32_to_f16((float)v);
+}
+static inline float e_to_f32(int elem, uint16_t a) { return elem == ORC_ELEM_BF16 ? orc_bf16_to_f32(a) : orc_f16_to_f32(a); }
+static inline uint16_t e_from_f32(int elem, float f) { return elem == ORC_ELEM_BF16 ? orc_f32_to_bf16(f) : orc_f32_to_f16(f); }
 /* Correctly rounded fused multiply-add on binary16, by exact integer arithmetic: every
  * finite half is an integer multiple of 2^-24, so a*b + c is an integer multiple of 2^-48
  * that fits in 128 bits.  Used for the reference converter's fma.rn.f16x2 and by tests
@@ -187,6 +231,18 @@ ORC_API void orc_h_mul_n(uint16_t *out, const uint16_t *a, const uint16_t *b, si
 ORC_API void orc_h_add_n(uint16_t *out, const uint16_t *a, const uint16_t *b, size_t n) {
   for (size_t i = 0; i < n; ++i) out[i] = h_add(a[i], b[i]);
 }
+ORC_API void orc_bf16_to_f32_n(float *out, const uint16_t *in, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = orc_bf16_to_f32(in[i]);
+}
+ORC_API void orc_f32_to_bf16_n(uint16_t *out, const float *in, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = orc_f32_to_bf16(in[i]);
+}
+ORC_API void orc_bf16_mul_n(uint16_t *out, const uint16_t *a, const uint16_t *b, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = b_mul(a[i], b[i]);
+}
+ORC_API void orc_bf16_add_n(uint16_t *out, const uint16_t *a, const uint16_t *b, size_t n) {
+  for (size_t i = 0; i < n; ++i) out[i] = b_add(a[i], b[i]);
+}
 ORC_API void orc_h_fma_n(uint16_t *out, const uint16_t *a, const uint16_t *b, const uint16_t *c, size_t n) {
   for (size_t i = 0; i < n; ++i) out[i] = orc_h_fma(a[i], b[i], c[i]);
 }
@@ -227,6 +283,11 @@ static inline int get_int4(const uint8_t *packed, size_t idx) {
 ORC_API void orc_fold_zero_points(uint16_t *out, const uint16_t *scales, const int8_t *zeros, size_t n) {
   for (size_t i = 0; i < n; ++i) {
     out[i] = h_mul(h_from_int(-(int)zeros[i]), scales[i]); /* preprocess.h:99 */
+  }
+}
+ORC_API void orc_fold_zero_points_bf16(uint16_t *out, const uint16_t *scales, const int8_t *zeros, size_t n) {
+  for (size_t i = 0; i < n; ++i) {
+    out[i] = b_mul(e_from_int(ORC_ELEM_BF16, -(int)zeros[i]), scales[i]); /* preprocess.h:99 with bfloat16_t */
   }
 }
 
@@ -312,15 +373,15 @@ ORC_API void orc_ref_convert_u8x4(uint16_t out[4], uint32_t w) {
 enum { ORC_ZERO_NONE = 0, ORC_ZERO_INT8 = 1, ORC_ZERO_FOLDED_F16 = 2 };
 enum { ORC_PER_COLUMN_SCALE_ONLY = 1, ORC_FINEGRAINED_SCALE_ONLY = 2, ORC_FINEGRAINED_SCALE_AND_ZEROS = 3 };
 
-static inline uint16_t dequant_one(int q, uint16_t s, int zero_kind, const void *zero, size_t zi) {
-  uint16_t p = h_mul(h_from_int(q), s); /* host/mixed_gemv.h:95-96 first product */
+static inline uint16_t dequant_one(int elem, int q, uint16_t s, int zero_kind, const void *zero, size_t zi) {
+  uint16_t p = e_mul(elem, e_from_int(elem, q), s); /* host/mixed_gemv.h:95-96 first product */
   if (zero_kind == ORC_ZERO_INT8) {
     /* host/mixed_gemv.h:92-93: scale_x_zero = -(s * half(z)) */
-    uint16_t sz = h_neg(h_mul(s, h_from_int((int)((const int8_t *)zero)[zi])));
-    return h_add(p, sz);
+    uint16_t sz = h_neg(e_mul(elem, s, e_from_int(elem, (int)((const int8_t *)zero)[zi])));
+    return e_add(elem, p, sz);
   } else if (zero_kind == ORC_ZERO_FOLDED_F16) {
     /* warp_dequantizer.h:57: plus(mul(q, s), zadd) */
-    return h_add(p, ((const uint16_t *)zero)[zi]);
+    return e_add(elem, p, ((const uint16_t *)zero)[zi]);
   }
   return p; /* warp_dequantizer.h:90 */
 }
@@ -332,7 +393,7 @@ static inline int get_q(const void *w, int bits, size_t idx) {
 /* W: un-preprocessed weights, [n_out][k] row-major, int4 packed two per byte or int8.
  * scale: [k/g][n_out] (n_out contiguous), per-column: [n_out].  zero: same shape, int8 or
  * fp16 according to zero_kind.  out: [n_out][k] fp16 bit patterns. */
-ORC_API int orc_dequantize(uint16_t *out, const void *W, const uint16_t *scale, const void *zero,
+static int dequantize_impl(int elem, uint16_t *out, const void *W, const uint16_t *scale, const void *zero,
                            int zero_kind, int n_out, int k, int group_size, int quant_op, int bits) {
   if (bits != 4 && bits != 8) return -1;
   if (quant_op == ORC_PER_COLUMN_SCALE_ONLY) group_size = k; /* mixed_gemv_test.cu:142-143 */
@@ -344,10 +405,20 @@ ORC_API int orc_dequantize(uint16_t *out, const void *W, const uint16_t *scale, 
       int g = kk / group_size; /* host/mixed_gemv.h:88 */
       size_t si = (size_t)g * (size_t)n_out + (size_t)n;
       int q = get_q(W, bits, (size_t)n * (size_t)k + (size_t)kk);
-      out[(size_t)n * (size_t)k + kk] = dequant_one(q, scale[si], zero_kind, zero, si);
+      out[(size_t)n * (size_t)k + kk] = dequant_one(elem, q, scale[si], zero_kind, zero, si);
     }
   }
   return 0;
+}
+
+ORC_API int orc_dequantize(uint16_t *out, const void *W, const uint16_t *scale, const void *zero,
+                           int zero_kind, int n_out, int k, int group_size, int quant_op, int bits) {
+  return dequantize_impl(ORC_ELEM_F16, out, W, scale, zero, zero_kind, n_out, k, group_size, quant_op, bits);
+}
+/* The same with bfloat16 scales / zeros / results (ORC_ZERO_FOLDED_F16 then means folded bf16). */
+ORC_API int orc_dequantize_bf16(uint16_t *out, const void *W, const uint16_t *scale, const void *zero,
+                                int zero_kind, int n_out, int k, int group_size, int quant_op, int bits) {
+  return dequantize_impl(ORC_ELEM_BF16, out, W, scale, zero, zero_kind, n_out, k, group_size, quant_op, bits);
 }
 
 /* ------------------------------------------------------------------------------------ */
@@ -357,7 +428,7 @@ ORC_API int orc_dequantize(uint16_t *out, const void *W, const uint16_t *scale, 
 /* mixed_gemv_test.cu:140).  threads <= 1 runs the reference's single-threaded loop.      */
 /* ------------------------------------------------------------------------------------ */
 
-static void gemv_rows(uint16_t *y, const void *W, const uint16_t *x, const uint16_t *scale,
+static void gemv_rows(int elem, uint16_t *y, const void *W, const uint16_t *x, const uint16_t *scale,
                       const void *zero, const uint16_t *bias, int zero_kind, int n_out,
                       int m_batch, int k, int group_size, int bits, int n_begin, int n_end) {
   for (int b = 0; b < m_batch; ++b) {
@@ -368,16 +439,16 @@ static void gemv_rows(uint16_t *y, const void *W, const uint16_t *x, const uint1
         int g = kk / group_size; /* :88 */
         size_t si = (size_t)g * (size_t)n_out + (size_t)n;
         int q = get_q(W, bits, (size_t)n * (size_t)k + (size_t)kk);
-        float dq = orc_f16_to_f32(dequant_one(q, scale[si], zero_kind, zero, si)); /* :92-96 */
-        acc += orc_f16_to_f32(xb[kk]) * dq; /* :98 */
+        float dq = e_to_f32(elem, dequant_one(elem, q, scale[si], zero_kind, zero, si)); /* :92-96 */
+        acc += e_to_f32(elem, xb[kk]) * dq; /* :98 */
       }
-      float bias_val = bias ? orc_f16_to_f32(bias[n]) : 0.0f; /* :102 */
-      y[(size_t)b * (size_t)n_out + n] = orc_f32_to_f16(acc + bias_val); /* :103, Identity activation */
+      float bias_val = bias ? e_to_f32(elem, bias[n]) : 0.0f; /* :102 */
+      y[(size_t)b * (size_t)n_out + n] = e_from_f32(elem, acc + bias_val); /* :103, Identity activation */
     }
   }
 }
 
-ORC_API int orc_gemv(uint16_t *y, const void *W, const uint16_t *x, const uint16_t *scale,
+static int gemv_impl(int elem, uint16_t *y, const void *W, const uint16_t *x, const uint16_t *scale,
                      const void *zero, const uint16_t *bias, int zero_kind, int n_out, int m_batch,
                      int k, int group_size, int quant_op, int bits, int threads) {
   if (bits != 4 && bits != 8) return -1;
@@ -386,7 +457,7 @@ ORC_API int orc_gemv(uint16_t *y, const void *W, const uint16_t *x, const uint16
   if (quant_op != ORC_FINEGRAINED_SCALE_AND_ZEROS) zero_kind = ORC_ZERO_NONE;
   if (group_size <= 0) return -1;
   if (threads <= 1) {
-    gemv_rows(y, W, x, scale, zero, bias, zero_kind, n_out, m_batch, k, group_size, bits, 0, n_out);
+    gemv_rows(elem, y, W, x, scale, zero, bias, zero_kind, n_out, m_batch, k, group_size, bits, 0, n_out);
     return 0;
   }
 #ifdef _OPENMP
@@ -394,9 +465,23 @@ ORC_API int orc_gemv(uint16_t *y, const void *W, const uint16_t *x, const uint16
 #endif
   for (int n0 = 0; n0 < n_out; n0 += 16) {
     int n1 = n0 + 16 < n_out ? n0 + 16 : n_out;
-    gemv_rows(y, W, x, scale, zero, bias, zero_kind, n_out, m_batch, k, group_size, bits, n0, n1);
+    gemv_rows(elem, y, W, x, scale, zero, bias, zero_kind, n_out, m_batch, k, group_size, bits, n0, n1);
   }
   return 0;
+}
+
+ORC_API int orc_gemv(uint16_t *y, const void *W, const uint16_t *x, const uint16_t *scale,
+                     const void *zero, const uint16_t *bias, int zero_kind, int n_out, int m_batch,
+                     int k, int group_size, int quant_op, int bits, int threads) {
+  return gemv_impl(ORC_ELEM_F16, y, W, x, scale, zero, bias, zero_kind, n_out, m_batch, k, group_size, quant_op, bits,
+                   threads);
+}
+/* The same loop with bfloat16 as ElementB / ElementScale / ElementOutput (host/mixed_gemv.h:24-31). */
+ORC_API int orc_gemv_bf16(uint16_t *y, const void *W, const uint16_t *x, const uint16_t *scale,
+                          const void *zero, const uint16_t *bias, int zero_kind, int n_out, int m_batch,
+                          int k, int group_size, int quant_op, int bits, int threads) {
+  return gemv_impl(ORC_ELEM_BF16, y, W, x, scale, zero, bias, zero_kind, n_out, m_batch, k, group_size, quant_op, bits,
+                   threads);
 }
 
 ORC_API int orc_max_threads(void) {

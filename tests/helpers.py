@@ -18,7 +18,10 @@ class Problem:
     """Raw (un-preprocessed) operands of one GEMV, as numpy arrays."""
 
     def __init__(self, tag, n_out, k, bits, quant_op, group_size, m_batch=1, bias=False, x_dist="uniform",
-                 scale_range=(0.001, 0.02), zero_kind="f16", zero_range=(-0.05, 0.05), buffer=0):
+                 scale_range=(0.001, 0.02), zero_kind="f16", zero_range=(-0.05, 0.05), buffer=0, element="f16"):
+        """element="bf16": the same draws rounded to bfloat16; x / scale / zero_add / bias are then
+        uint16 arrays of bf16 bit patterns (numpy has no such dtype)."""
+        self.element = element
         self.tag, self.n_out, self.k, self.bits, self.quant_op = tag, n_out, k, bits, quant_op
         self.group_size = k if quant_op == PER_COLUMN else group_size
         self.m_batch = m_batch
@@ -41,13 +44,26 @@ class Problem:
                 self.zero_add = orc.fill_uniform_f16(groups * n_out, seed_of(tag, "z", buffer), *zero_range).reshape(
                     groups, n_out)
         self.bias = orc.fill_uniform_f16(n_out, seed_of(tag, "b"), -0.1, 0.1) if bias else None
+        if element == "bf16":
+            to_bf16 = lambda a: None if a is None else orc.f32_to_bf16_array(a.astype(np.float32))  # noqa: E731
+            self.x, self.scale, self.bias = to_bf16(self.x), to_bf16(self.scale), to_bf16(self.bias)
+            if self.zeros_i8 is not None:
+                self.zero_add = orc.fold_zero_points_bf16(self.scale, self.zeros_i8)
+            else:
+                self.zero_add = to_bf16(self.zero_add)
 
     def oracle_dequant(self):
+        if self.element == "bf16":
+            return orc.dequantize_bf16(self.w_raw, self.scale, self.zero_add, self.n_out, self.k, self.group_size,
+                                       self.quant_op, self.bits)
         return orc.dequantize(self.w_raw, self.scale, self.zero_add, self.n_out, self.k, self.group_size,
                               self.quant_op, self.bits)
 
     def oracle_gemv(self, threads=8, literal_int8_zero=False):
         zero = self.zeros_i8 if (literal_int8_zero and self.zeros_i8 is not None) else self.zero_add
+        if self.element == "bf16":
+            return orc.gemv_bf16(self.w_raw, self.x, self.scale, zero, self.bias, self.n_out, self.m_batch, self.k,
+                                 self.group_size, self.quant_op, self.bits, threads=threads)
         return orc.gemv(self.w_raw, self.x, self.scale, zero, self.bias, self.n_out, self.m_batch, self.k,
                         self.group_size, self.quant_op, self.bits, threads=threads)
 
@@ -75,6 +91,21 @@ def error_report(got, ref):
     return float(abs_err.max(initial=0.0)), float(rel.max(initial=0.0)), floor
 
 
+def bf16_ulp_report(got_bits, ref_bits):
+    """For bf16 outputs (uint16 bit patterns): the largest |got - ref| in units of the bf16 ulp of
+    max(|ref|, 2^-7 * rms(ref)), and the fraction of outputs whose bits differ.  One ulp is 2^-7
+    relative at the bottom of a binade, so "within 2e-3" cannot be asked of a bf16 result: two
+    correct fp32 sums that differ in their last bits can round to adjacent bf16 values."""
+    g = orc.bf16_to_f32_array(got_bits).astype(np.float64).reshape(-1)
+    r = orc.bf16_to_f32_array(ref_bits).astype(np.float64).reshape(-1)
+    rms = float(np.sqrt(np.mean(r * r))) if r.size else 0.0
+    floor = max(rms * REL_FLOOR_FRACTION, 2.0 ** -100)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(r), floor))) - 7)
+    worst = float((np.abs(g - r) / ulp).max(initial=0.0))
+    differing = float(np.mean(np.asarray(got_bits).reshape(-1) != np.asarray(ref_bits).reshape(-1)))
+    return worst, differing
+
+
 class DeviceProblem:
     """Uploads a Problem through the library's own preprocessor."""
 
@@ -97,15 +128,18 @@ class DeviceProblem:
         p = self.p
         self.y.fill_(0x7e00)  # NaN pattern: every output must be overwritten
         mg.device_gemv(self.w, self.x, self.scale, self.zero, self.bias, self.y, 1, p.n_out, p.m_batch, p.k,
-                       p.group_size, p.quant_op, p.bits)
+                       p.group_size, p.quant_op, p.bits, element=p.element)
         torch.cuda.synchronize()
-        return self.y.cpu().numpy().view(np.float16)
+        out = self.y.cpu().numpy()
+        return out.view(np.uint16) if p.element == "bf16" else out.view(np.float16)
 
     def dequant(self):
         import torch
         import mixed_gemv_amd as mg
         p = self.p
         out = torch.zeros((p.n_out, p.k), dtype=torch.int16, device=self.w.device)
-        mg.dequantize(self.w, self.scale, self.zero, out, p.n_out, p.k, p.group_size, p.quant_op, p.bits)
+        mg.dequantize(self.w, self.scale, self.zero, out, p.n_out, p.k, p.group_size, p.quant_op, p.bits,
+                      element=p.element)
         torch.cuda.synchronize()
-        return out.cpu().numpy().view(np.float16)
+        out = out.cpu().numpy()
+        return out.view(np.uint16) if p.element == "bf16" else out.view(np.float16)

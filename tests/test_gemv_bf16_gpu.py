@@ -1,0 +1,180 @@
+"""GPU parity of the bfloat16 entry points (mgemv_gemv_bf16, mgemv_dequantize_bf16), called
+through the C-ABI, against the CPU oracle's bf16 functions.
+
+Bars: dequantised weights bit-exact.  Outputs: the oracle's bf16 value or one of its two
+neighbours (1 ulp; two correct fp32 sums that differ in their last bits can round to adjacent
+bf16 values, and a bf16 ulp is up to 2^-7 relative, so the fp16 bar of 2e-3 cannot be asked),
+with at most 1 % of the outputs differing at all."""
+import numpy as np
+import pytest
+
+import mixed_gemv_amd as mg
+import oracle as orc
+from helpers import PER_COLUMN, SCALE_AND_ZEROS, SCALE_ONLY, DeviceProblem, Problem, bf16_ulp_report
+
+pytestmark = pytest.mark.gpu
+
+MAX_ULP = 1.0 + 1e-6
+MAX_DIFFERING = 0.01
+
+
+def check(prob, gpu, dequant=True):
+    dev = DeviceProblem(prob, gpu)
+    if dequant:
+        mism = int((dev.dequant() != prob.oracle_dequant()).sum())
+        assert mism == 0, f"{mism} dequantised weights differ"
+    y = dev.run()
+    ref = prob.oracle_gemv(threads=16)
+    ulp, differing = bf16_ulp_report(y, ref)
+    print(f"{prob.tag}: worst {ulp:.3f} ulp, {100 * differing:.2f} % of outputs differ", flush=True)
+    assert np.isfinite(orc.bf16_to_f32_array(y)).all()
+    assert ulp <= MAX_ULP and differing <= MAX_DIFFERING
+    return dev, y
+
+
+SMALL = [
+    # tag, n_out, k, bits, quant_op, group, m_batch, bias
+    ("b_i4_sz_g128", 256, 1024, 4, SCALE_AND_ZEROS, 128, 1, False),
+    ("b_i4_sz_g64", 256, 1024, 4, SCALE_AND_ZEROS, 64, 1, True),
+    ("b_i4_sz_g256", 64, 2048, 4, SCALE_AND_ZEROS, 256, 2, True),
+    ("b_i4_s_g128", 128, 2048, 4, SCALE_ONLY, 128, 1, True),
+    ("b_i4_col", 128, 1024, 4, PER_COLUMN, 0, 3, False),
+    ("b_i8_col", 256, 1024, 8, PER_COLUMN, 0, 1, True),
+    ("b_i8_sz_g64", 128, 512, 8, SCALE_AND_ZEROS, 64, 4, False),
+    ("b_i8_s_g96", 32, 576, 8, SCALE_ONLY, 96, 1, False),           # group not a power of two
+    ("b_i4_ragged", 100, 1120, 4, SCALE_AND_ZEROS, 160, 1, True),   # n_out % 16 != 0, k % 512 != 0, odd group
+    ("b_i4_tiny", 4, 64, 4, SCALE_AND_ZEROS, 64, 1, True),
+    ("b_i4_mb7", 64, 1024, 4, SCALE_AND_ZEROS, 64, 7, False),       # two launches of the VALU kernel
+    ("b_i8_mb16", 48, 512, 8, PER_COLUMN, 0, 16, True),
+]
+
+
+@pytest.mark.parametrize("cfg", SMALL, ids=[c[0] for c in SMALL])
+@pytest.mark.parametrize("form", ["auto", "general"])
+def test_small_parity(gpu, cfg, form):
+    tag, n_out, k, bits, qop, g, mb, bias = cfg
+    try:
+        mg.set_dequant_form(mg.DEQUANT_EXACT_INTEGER if form == "general" else mg.DEQUANT_AUTO)
+        check(Problem(tag, n_out, k, bits, qop, g, m_batch=mb, bias=bias, element="bf16"), gpu)
+    finally:
+        mg.set_dequant_form(mg.DEQUANT_AUTO)
+
+
+@pytest.mark.parametrize("form", ["auto", "general"])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_dequant_every_finite_scale_bit_exact(gpu, bits, form):
+    """Each (row, group) gets its own scale so that ALL finite bf16 scales (subnormals, huge values,
+    both signs) meet every int4 weight value (a spread of int8 values), with an additive zero:
+    multiply, round, add, round.  Consecutive bit patterns share a tile, so in "auto" the tiles
+    whose scales all lie in 0x0001..0x7aff take the fused form and the others the general one."""
+    allbits = np.arange(65536, dtype=np.uint16)
+    finite = allbits[(allbits & 0x7F80) != 0x7F80]            # 65280 values
+    n_out, g = 64, 64
+    groups = finite.size // n_out                              # 1020
+    k = groups * g
+    prob = Problem(f"b_allscales{bits}", n_out, k, bits, SCALE_AND_ZEROS, g, element="bf16")
+    if bits == 4:   # every group of every row holds all 16 values
+        q = np.tile(np.arange(-8, 8, dtype=np.int8), n_out * k // 16)
+        prob.q, prob.w_raw = q, orc.pack_int4(q)
+    prob.scale = finite.reshape(groups, n_out).copy()
+    zero = orc.f32_to_bf16_array(orc.fill_uniform_f16(groups * n_out, 99, -0.05, 0.05).astype(np.float32)).reshape(groups, n_out)
+    zero[::7, ::3] = 0x0000
+    zero[1::7, ::5] = 0x8000
+    zero[2::11, :] = np.arange(1, n_out + 1, dtype=np.uint16)          # subnormal additive terms
+    prob.zero_add = zero
+    try:
+        mg.set_dequant_form(mg.DEQUANT_EXACT_INTEGER if form == "general" else mg.DEQUANT_AUTO)
+        got = DeviceProblem(prob, gpu).dequant()
+    finally:
+        mg.set_dequant_form(mg.DEQUANT_AUTO)
+    want = prob.oracle_dequant()
+    nan = np.isnan(orc.bf16_to_f32_array(want))
+    assert np.array_equal(np.isnan(orc.bf16_to_f32_array(got)), nan)   # inf - inf: NaN on both sides
+    assert int((got[~nan] != want[~nan]).sum()) == 0
+
+
+def test_one_hot_activation_is_bit_exact_through_the_gemv_kernel(gpu):
+    """y[n] == dq[n, j] bit for bit (up to the sign of a zero): pins the dequantiser inside the GEMV kernel."""
+    prob = Problem("b_onehot", 96, 1536, 4, SCALE_AND_ZEROS, 128, element="bf16")
+    dq = prob.oracle_dequant()
+    dev = DeviceProblem(prob, gpu)
+    import torch
+    for j in (0, 1, 127, 128, 511, 512, 1000, 1535):
+        x = np.zeros((1, prob.k), dtype=np.uint16)
+        x[0, j] = 0x3F80
+        dev.x = torch.from_numpy(x.view(np.int16)).to(gpu)
+        y = dev.run()[0]
+        nz = (dq[:, j] & 0x7FFF) != 0
+        assert np.array_equal(y[nz], dq[:, j][nz]), j
+        assert np.all((y[~nz] & 0x7FFF) == 0), j
+
+
+def test_split_k_and_tile_walk_invariance(gpu):
+    prob = Problem("b_splitk", 192, 8192, 4, SCALE_AND_ZEROS, 128, bias=True, x_dist="normal", element="bf16")
+    dev = DeviceProblem(prob, gpu)
+    ref = prob.oracle_gemv(threads=16)
+    results = {}
+    try:
+        for sk, tw, cap in ((1, 1, 0), (1, 4, 0), (2, 2, 0), (4, 2, 0), (8, 1, 0), (1, 1, 5), (4, 2, 2)):
+            mg.set_launch_override(sk, tw, 0, cap)
+            a = dev.run().copy()
+            assert np.array_equal(a, dev.run()), "same launch geometry must be bit-reproducible"
+            ulp, differing = bf16_ulp_report(a, ref)
+            assert ulp <= MAX_ULP and differing <= MAX_DIFFERING, (sk, tw, cap, ulp, differing)
+            results[(sk, tw, cap)] = a
+    finally:
+        mg.set_launch_override(0, 0, 0, 0)
+    for other in ((1, 4, 0), (1, 1, 5)):   # the same k split adds in the same order wherever the tiles run
+        assert np.array_equal(results[(1, 1, 0)], results[other]), other
+
+
+def test_batched_launch_with_strides(gpu):
+    """batch_count problems in one launch: stacked weights and scales, shared activations."""
+    import torch
+    n_out, k, g, batch = 64, 1024, 128, 3
+    probs = [Problem(f"b_batch{b}", n_out, k, 4, SCALE_AND_ZEROS, g, bias=True, element="bf16") for b in range(batch)]
+    devs = [DeviceProblem(p, gpu) for p in probs]
+    w = torch.stack([d.w for d in devs]).contiguous()
+    s = torch.stack([d.scale for d in devs]).contiguous()
+    z = torch.stack([d.zero for d in devs]).contiguous()
+    bias = torch.stack([d.bias for d in devs]).contiguous()
+    y = torch.zeros((batch, 1, n_out), dtype=torch.int16, device=gpu)
+    mg.device_gemv(w, devs[0].x, s, z, bias, y, batch, n_out, 1, k, g, SCALE_AND_ZEROS, 4,
+                   batch_strides=(w.stride(0), 0, s.stride(0), bias.stride(0), y.stride(0)), element="bf16")
+    torch.cuda.synchronize()
+    got = y.cpu().numpy().view(np.uint16)
+    for b, p in enumerate(probs):
+        p.x = probs[0].x
+        ulp, differing = bf16_ulp_report(got[b], p.oracle_gemv(threads=8))
+        assert ulp <= MAX_ULP and differing <= MAX_DIFFERING
+
+
+def test_torch_bfloat16_tensors_select_the_bf16_entry_points(gpu):
+    import torch
+    prob = Problem("b_torch", 128, 1024, 4, SCALE_AND_ZEROS, 128, bias=True, element="bf16")
+    dev = DeviceProblem(prob, gpu)
+    want = dev.run()
+    x, s, z, b = (t.view(torch.bfloat16) for t in (dev.x, dev.scale, dev.zero, dev.bias))
+    y = torch.zeros((1, 128), dtype=torch.bfloat16, device=gpu)
+    mg.device_gemv(dev.w, x, s, z, b, y, 1, 128, 1, 1024, 128, SCALE_AND_ZEROS, 4)      # element from the dtype
+    torch.cuda.synchronize()
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), want)
+    adaptor = mg.GemvAdaptor(SCALE_AND_ZEROS, 4)
+    y.zero_()
+    adaptor(mg.GemvAdaptor.Arguments((128, 1, 1024), dev.w, x, s, z, b, y, group_size=128))
+    torch.cuda.synchronize()
+    assert np.array_equal(y.view(torch.int16).cpu().numpy().view(np.uint16), want)
+
+
+FULL = [
+    ("b_ns", 4096, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "uniform"),
+    ("b_c1", 4096, 4096, 8, PER_COLUMN, 0, 1, True, "uniform"),
+    ("b_c3a", 11008, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal"),
+    ("b_c4_m4", 8192, 8192, 4, SCALE_AND_ZEROS, 64, 4, True, "uniform"),
+]
+
+
+@pytest.mark.parametrize("cfg", FULL, ids=[c[0] for c in FULL])
+def test_baseline_shapes_full_size(gpu, cfg):
+    tag, n_out, k, bits, qop, g, mb, bias, xd = cfg
+    check(Problem(tag, n_out, k, bits, qop, g, m_batch=mb, bias=bias, x_dist=xd, element="bf16"), gpu)
