@@ -190,6 +190,7 @@ __device__ __forceinline__ void settle_dot_chain(float& acc) { asm volatile("s_n
 //            a zero product as the reference's multiply gives it.
 // ---------------------------------------------------------------------------------------------
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kActF16 = 0;

@@ -641,7 +641,7 @@ __device__ __forceinline__ u32x4 mfma_operand(const LdsActivations<BITS>& xa, in
   return *reinterpret_cast<const u32x4*>(xa.lane_base + (i * G::kChunkK + j * 8) * 2);
 }
 
-template <int BITS, int QOP, int GROUPS_PER_RUN, bool SHORT, typename Activations>
+template <int BITS, int QOP, int GROUPS_PER_RUN, bool SHORT, int ACT, typename Activations>
 __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
                                                        const Activations& xa, const ConvertRegs& c,
                                                        half2_t col_scale2) {
@@ -649,6 +649,28 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i) {
     const int gi = i * GROUPS_PER_RUN / kBlocksPerUnit;
+    if constexpr (ACT == kActBf16) {
+      // bf16: the same dequantiser as the VALU kernel (SHORT = fused form), v_mfma_f32_16x16x32_bf16
+      const uint32_t s_bits = QOP != MGEMV_PER_COLUMN_SCALE_ONLY ? f.s[gi] : as_u32(col_scale2);
+      const Bf16Scale bs = make_bf16_scale<BITS, SHORT>(s_bits, kHasZero ? f.z[gi] : 0u);
+#pragma unroll
+      for (int j = 0; j < (BITS == 4 ? 4 : 2); ++j) {
+        u32x4 a;
+        if constexpr (BITS == 4) {
+          uint32_t d[4];
+          dequant_int4_word_bf16<kHasZero, SHORT>(f.w[i][j], c, bs, d);
+          a = u32x4{d[0], d[1], d[2], d[3]};
+        } else {
+          uint32_t d0[2], d1[2];
+          dequant_int8_word_bf16<kHasZero, SHORT>(f.w[i][2 * j], bs, d0);
+          dequant_int8_word_bf16<kHasZero, SHORT>(f.w[i][2 * j + 1], bs, d1);
+          a = u32x4{d0[0], d0[1], d1[0], d1[1]};
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                      __builtin_bit_cast(bf16x8_t, mfma_operand<BITS>(xa, i, j)), acc, 0, 0, 0);
+      }
+      continue;
+    }
     half2_t s2 = col_scale2, z2 = half2_t{};
     if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) s2 = splat_low(f.s[gi]);
     if constexpr (kHasZero) z2 = splat_low(f.z[gi]);
@@ -690,19 +712,19 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
   }
 }
 
-template <int BITS, int QOP, int GROUPS_PER_RUN, typename Activations>
+template <int BITS, int QOP, int GROUPS_PER_RUN, int ACT = kActF16, typename Activations>
 __device__ __forceinline__ void compute_unit_mfma(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
                                                   const Activations& xa, const ConvertRegs& c,
                                                   half2_t col_scale2, bool short_allowed) {
-  if constexpr (BITS == 4) {
+  if constexpr (BITS == 4 || ACT == kActBf16) {
     bool take_short = short_allowed;
-    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form<kActF16>(f.s);
+    if constexpr (QOP != MGEMV_PER_COLUMN_SCALE_ONLY) take_short = take_short && wave_scales_permit_short_form<ACT>(f.s);
     if (take_short) {
-      compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, true>(acc, f, xa, c, col_scale2);
+      compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, true, ACT>(acc, f, xa, c, col_scale2);
       return;
     }
   }
-  compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, false>(acc, f, xa, c, col_scale2);
+  compute_unit_mfma_form<BITS, QOP, GROUPS_PER_RUN, false, ACT>(acc, f, xa, c, col_scale2);
 }
 
 // blockDim = (64 * split_k, tiles_per_wg); each wave works on T consecutive tiles so that the
@@ -931,7 +953,7 @@ __device__ __forceinline__ void park_x_rows(const XRows<BITS, ROUNDS>& r, uint8_
 // blockDim = (64 * split_k, tiles_per_wg), at most 8 waves.  Dynamic LDS: split_k * 2 stages of
 // (ROUNDS * tiles_per_wg) rows x kRowStride bytes, then tiles_per_wg * split_k * 256 floats for
 // the split-K combine.
-template <int BITS, int QOP, int GROUPS_PER_RUN, int ROUNDS>
+template <int BITS, int QOP, int GROUPS_PER_RUN, int ROUNDS, int ACT>
 __global__ void __launch_bounds__(kWave * kMaxWavesPerMfmaWorkgroup)
 gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out,
                      int k, uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
@@ -1000,7 +1022,7 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
   if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
     col_scale = splat(p.scale[row]);
     const uint32_t bits[1] = {as_u32(col_scale)};
-    short_ok = short_ok && wave_scales_permit_short_form<kActF16>(bits);
+    short_ok = short_ok && wave_scales_permit_short_form<ACT>(bits);
   }
   const ConvertRegs c = make_convert_regs();
 
@@ -1019,7 +1041,7 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
     __builtin_amdgcn_sched_barrier(0);
     if (u < units) {
       const LdsActivations<BITS> xa{my_stages + operand_offset};
-      compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc, wa, xa, c, col_scale, short_ok);
+      compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, wa, xa, c, col_scale, short_ok);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (u + 1 < steps) {
@@ -1031,7 +1053,7 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
       __builtin_amdgcn_sched_barrier(0);
       if (u + 1 < units) {
         const LdsActivations<BITS> xa{my_stages + stage_bytes + operand_offset};
-        compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN>(acc, wb, xa, c, col_scale, short_ok);
+        compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, wb, xa, c, col_scale, short_ok);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1058,8 +1080,13 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
       const int n = n0 + v;
       if (n < p.n_out) {
         float r = sum[v];
-        if (has_bias) r += (float)tail.bias[n];
-        tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
+        if constexpr (ACT == kActBf16) {
+          if (has_bias) r += bf16_low_to_f32(reinterpret_cast<const uint16_t*>(tail.bias)[n]);
+          reinterpret_cast<uint16_t*>(tail.y)[(size_t)m * (size_t)p.n_out + n] = (uint16_t)pack_bf16(r, 0.0f);
+        } else {
+          if (has_bias) r += (float)tail.bias[n];
+          tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
+        }
       }
     }
   }
@@ -1498,9 +1525,9 @@ hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr) {
 }
 
 // LDS-staged matrix-core kernel: 2 tiles per workgroup share the activation stage.
-template <int BITS, int QOP, int GPR, int ROUNDS>
+template <int BITS, int QOP, int GPR, int ROUNDS, int ACT>
 hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
-  const auto kernel = gemv_mfma_lds_kernel<BITS, QOP, GPR, ROUNDS>;
+  const auto kernel = gemv_mfma_lds_kernel<BITS, QOP, GPR, ROUNDS, ACT>;
   if (g.lds > 48 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds);
@@ -1511,37 +1538,44 @@ hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
                 pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
 }
 
-template <int BITS, int QOP, int GPR>
+template <int BITS, int QOP, int GPR, int ACT>
 hipError_t launch_mfma_lds_kernel(const GemvLaunch& g, int rounds) {
-  return rounds == 4 ? launch_mfma_lds_kernel_r<BITS, QOP, GPR, 4>(g) : launch_mfma_lds_kernel_r<BITS, QOP, GPR, 8>(g);
+  return rounds == 4 ? launch_mfma_lds_kernel_r<BITS, QOP, GPR, 4, ACT>(g)
+                     : launch_mfma_lds_kernel_r<BITS, QOP, GPR, 8, ACT>(g);
 }
 
-template <int BITS, int QOP>
+template <int BITS, int QOP, int ACT>
 hipError_t launch_mfma_lds_gpr(const GemvLaunch& g, int gpr, int rounds) {
   if constexpr (QOP == MGEMV_PER_COLUMN_SCALE_ONLY) {
-    return launch_mfma_lds_kernel<BITS, QOP, 1>(g, rounds);
+    return launch_mfma_lds_kernel<BITS, QOP, 1, ACT>(g, rounds);
   } else {
     switch (gpr) {
-      case 1: return launch_mfma_lds_kernel<BITS, QOP, 1>(g, rounds);
-      case 2: return launch_mfma_lds_kernel<BITS, QOP, 2>(g, rounds);
-      default: return launch_mfma_lds_kernel<BITS, QOP, 4>(g, rounds);
+      case 1: return launch_mfma_lds_kernel<BITS, QOP, 1, ACT>(g, rounds);
+      case 2: return launch_mfma_lds_kernel<BITS, QOP, 2, ACT>(g, rounds);
+      default: return launch_mfma_lds_kernel<BITS, QOP, 4, ACT>(g, rounds);
     }
   }
 }
 
-hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds) {
+template <int ACT>
+hipError_t launch_mfma_lds_act(const GemvLaunch& g, int bits, int qop, int gpr, int rounds) {
   if (bits == 4) {
     switch (qop) {
-      case 1: return launch_mfma_lds_gpr<4, 1>(g, gpr, rounds);
-      case 2: return launch_mfma_lds_gpr<4, 2>(g, gpr, rounds);
-      default: return launch_mfma_lds_gpr<4, 3>(g, gpr, rounds);
+      case 1: return launch_mfma_lds_gpr<4, 1, ACT>(g, gpr, rounds);
+      case 2: return launch_mfma_lds_gpr<4, 2, ACT>(g, gpr, rounds);
+      default: return launch_mfma_lds_gpr<4, 3, ACT>(g, gpr, rounds);
     }
   }
   switch (qop) {
-    case 1: return launch_mfma_lds_gpr<8, 1>(g, gpr, rounds);
-    case 2: return launch_mfma_lds_gpr<8, 2>(g, gpr, rounds);
-    default: return launch_mfma_lds_gpr<8, 3>(g, gpr, rounds);
+    case 1: return launch_mfma_lds_gpr<8, 1, ACT>(g, gpr, rounds);
+    case 2: return launch_mfma_lds_gpr<8, 2, ACT>(g, gpr, rounds);
+    default: return launch_mfma_lds_gpr<8, 3, ACT>(g, gpr, rounds);
   }
+}
+
+hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act) {
+  return act == kActBf16 ? launch_mfma_lds_act<kActBf16>(g, bits, qop, gpr, rounds)
+                         : launch_mfma_lds_act<kActF16>(g, bits, qop, gpr, rounds);
 }
 
 template <int BITS, int ACT>
@@ -1578,8 +1612,11 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
   g.group_size = group_size;
   PlanKnobs knobs = knobs_for(n_out, k, weight_bits, group_size, m_batch);
   if (act == kActBf16) {
-    knobs.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1;  // bf16: VALU kernel only, ...
-    knobs.wide_waves = true;                              // ... whose fp32 dequantiser wants the registers of 8-wave workgroups
+    // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
+    // fp32 dequantiser wants the registers of 8-wave workgroups
+    if (num_tiles(n_out) < 2) knobs.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1;
+    knobs.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
+    knobs.wide_waves = true;
   }
   g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs);
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
@@ -1609,7 +1646,7 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
       const int row_stride = step_k(weight_bits) * 2 + 16;
       g.lds = (size_t)g.plan.split_k * 2 * g.plan.staged_rows * row_stride +
               (g.plan.split_k > 1 ? (size_t)g.plan.tiles_per_wg * g.plan.split_k * kWave * 4 * sizeof(float) : 0);
-      return launch_mfma_lds(g, weight_bits, quant_op, gpr, g.plan.staged_rows / g.plan.tiles_per_wg) == hipSuccess
+      return launch_mfma_lds(g, weight_bits, quant_op, gpr, g.plan.staged_rows / g.plan.tiles_per_wg, act) == hipSuccess
                  ? MGEMV_OK
                  : MGEMV_ERR_LAUNCH;
     }

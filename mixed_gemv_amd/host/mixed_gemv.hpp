@@ -39,6 +39,9 @@ constexpr bool hasZero(WeightOnlyQuantOp op) { return op == WeightOnlyQuantOp::F
 // utils/type_base.h:7-16
 enum class QuantType { W8_A16 = 0, W4_A16 = 1, W4_AFP8 = 2 };
 enum class LayoutType { kRowMajor = 0, kColumnMajor = 1 };
+// The reference's ElementB = ElementScale = ElementOutput template arguments (host/mixed_gemv.h:24-31):
+// what the 16-bit operands (typed half_t below) hold.
+enum class ElementType { kFloat16 = 0, kBFloat16 = 1 };
 
 class Error : public std::runtime_error {
  public:
@@ -72,8 +75,12 @@ struct SubBytePacker {
 
 // utils/preprocess.h:88-102
 struct ZeroPointPreprocessor {
-  static void neg_zero_point_multiplies_scale(half_t* neg_zeros_x_scales, const half_t* scales, const int8_t* zeros, int n) {
-    check(mgemv_fold_zero_points(neg_zeros_x_scales, scales, zeros, static_cast<size_t>(n)), "ZeroPointPreprocessor");
+  static void neg_zero_point_multiplies_scale(half_t* neg_zeros_x_scales, const half_t* scales, const int8_t* zeros, int n,
+                                              ElementType element = ElementType::kFloat16) {
+    check(element == ElementType::kBFloat16
+              ? mgemv_fold_zero_points_bf16(neg_zeros_x_scales, scales, zeros, static_cast<size_t>(n))
+              : mgemv_fold_zero_points(neg_zeros_x_scales, scales, zeros, static_cast<size_t>(n)),
+          "ZeroPointPreprocessor");
   }
 };
 
@@ -126,8 +133,9 @@ class GemvAdaptor {
     long long batch_stride_B = 0, batch_stride_scale = 0, batch_stride_C = 0, batch_stride_D = 0;  // elements
   };
 
-  GemvAdaptor(WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4)
-      : quant_op_(quant_op), weight_bits_(weight_bits) {}
+  GemvAdaptor(WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4,
+              ElementType element = ElementType::kFloat16)
+      : quant_op_(quant_op), weight_bits_(weight_bits), element_(element) {}
 
   void initialize(const Arguments& args, void* /*stream*/ = nullptr) {
     // gemv_adaptor.h:199-203
@@ -140,10 +148,11 @@ class GemvAdaptor {
     if (!initialized_) throw std::logic_error("GemvAdaptor::run before initialize");
     const Arguments& a = args_;
     const half_t* zero = hasZero(quant_op_) ? a.ref_zero_point.ptr : nullptr;  // mixed_gemv_test.cu:145-147
-    check(mgemv_gemv_batched(a.ref_A.ptr, a.ref_B.ptr, a.ref_scale.ptr, zero, a.ref_C.ptr, a.ref_D.ptr, a.batch_count,
-                             a.problem_size.m(), a.problem_size.n(), a.problem_size.k(), a.group_size,
-                             static_cast<int>(quant_op_), weight_bits_, a.batch_stride_A, a.batch_stride_B,
-                             a.batch_stride_scale, a.batch_stride_C, a.batch_stride_D, stream),
+    const auto gemv = element_ == ElementType::kBFloat16 ? mgemv_gemv_batched_bf16 : mgemv_gemv_batched;
+    check(gemv(a.ref_A.ptr, a.ref_B.ptr, a.ref_scale.ptr, zero, a.ref_C.ptr, a.ref_D.ptr, a.batch_count,
+               a.problem_size.m(), a.problem_size.n(), a.problem_size.k(), a.group_size,
+               static_cast<int>(quant_op_), weight_bits_, a.batch_stride_A, a.batch_stride_B,
+               a.batch_stride_scale, a.batch_stride_C, a.batch_stride_D, stream),
           "GemvAdaptor::run");
   }
 
@@ -155,6 +164,7 @@ class GemvAdaptor {
  private:
   WeightOnlyQuantOp quant_op_;
   int weight_bits_;
+  ElementType element_;
   Arguments args_{};
   bool initialized_ = false;
 };
@@ -164,7 +174,7 @@ class GemvAdaptor {
 inline void device_gemv(const void* ptr_A, const half_t* ptr_B, const half_t* ptr_scale, const half_t* ptr_zero_point,
                         const half_t* ptr_C, half_t* ptr_D, int B, int M, int N, int K, int group_size,
                         WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4,
-                        void* stream = nullptr) {
+                        void* stream = nullptr, ElementType element = ElementType::kFloat16) {
   if (quant_op == WeightOnlyQuantOp::PER_COLUMN_SCALE_ONLY) group_size = K;            // :142-143
   if (quant_op != WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS) ptr_zero_point = nullptr;  // :145-147
   GemvAdaptor::Arguments args;
@@ -177,7 +187,7 @@ inline void device_gemv(const void* ptr_A, const half_t* ptr_B, const half_t* pt
   args.ref_D = {ptr_D, M};
   args.group_size = group_size;
   args.batch_count = B;
-  GemvAdaptor op(quant_op, weight_bits);
+  GemvAdaptor op(quant_op, weight_bits, element);
   op.initialize(args);
   op.run(stream);
 }

@@ -128,6 +128,38 @@ def test_split_k_and_tile_walk_invariance(gpu):
         assert np.array_equal(results[(1, 1, 0)], results[other]), other
 
 
+@pytest.mark.parametrize("bits,qop,g", [(4, SCALE_AND_ZEROS, 128), (4, SCALE_ONLY, 64), (4, PER_COLUMN, 0),
+                                        (8, SCALE_AND_ZEROS, 64), (8, PER_COLUMN, 0), (4, SCALE_AND_ZEROS, 160)])
+def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
+    """The same batches through the LDS-staged matrix-core kernel (v_mfma_f32_16x16x32_bf16) at
+    several k splits and through the VALU kernel (threshold forced), ragged shape, every mode,
+    both dequantiser forms."""
+    n_out, k = 100, 1120 if g in (0, 160) else 1024
+    for m_batch in (1, 5, 8, 13, 16):
+        prob = Problem(f"b_mc{bits}{qop}", n_out, k, bits, qop, g, m_batch=m_batch, bias=True, element="bf16")
+        dev = DeviceProblem(prob, gpu)
+        ref = prob.oracle_gemv(threads=8)
+        results = []
+        try:
+            for form in (mg.DEQUANT_AUTO, mg.DEQUANT_EXACT_INTEGER):
+                mg.set_dequant_form(form)
+                mg.set_matrix_core_threshold(1)
+                for split in (0, 1, 2):
+                    mg.set_launch_override(split, 0, 0, 0)
+                    results.append(dev.run().copy())
+                    assert np.array_equal(results[-1], dev.run())   # reproducible
+                mg.set_launch_override(0, 0, 0, 0)
+                mg.set_matrix_core_threshold(17)
+                results.append(dev.run().copy())   # VALU kernel
+        finally:
+            mg.set_matrix_core_threshold(0)
+            mg.set_launch_override(0, 0, 0, 0)
+            mg.set_dequant_form(mg.DEQUANT_AUTO)
+        for y in results:
+            ulp, differing = bf16_ulp_report(y, ref)
+            assert ulp <= MAX_ULP and differing <= MAX_DIFFERING, (m_batch, ulp, differing)
+
+
 def test_batched_launch_with_strides(gpu):
     """batch_count problems in one launch: stacked weights and scales, shared activations."""
     import torch
@@ -171,6 +203,7 @@ FULL = [
     ("b_c1", 4096, 4096, 8, PER_COLUMN, 0, 1, True, "uniform"),
     ("b_c3a", 11008, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal"),
     ("b_c4_m4", 8192, 8192, 4, SCALE_AND_ZEROS, 64, 4, True, "uniform"),
+    ("b_c4_m16", 8192, 8192, 4, SCALE_AND_ZEROS, 64, 16, True, "uniform"),   # matrix cores
 ]
 
 
