@@ -183,9 +183,10 @@ __device__ __forceinline__ void settle_dot_chain(float& acc) { asm volatile("s_n
 // Values are kept as packed pairs of bf16 bit patterns, (low, high) = ascending k.
 //
 // Two forms, as for fp16.  With 8u (int4) or u (int8) from v_cvt_f32_ubyteN:
-//   fused    fma(8u, s/8, -8s) resp. fma(u, s, -128s): exact, hence = q*s, for 0 < s < 2^119
-//            (s/8 never underflows the fp32 subnormals, -8s / -128s stays finite; for s > 0 a zero
-//            product is +0 on both routes);
+//   fused    fma(8u, s/8, -8s) resp. fma(u, s, -128s): exact, hence = q*s, for 2^-100 <= s < 2^119
+//            (-8s / -128s stays finite; for s > 0 a zero product is +0 on both routes).  For int4
+//            the fma and the conversions around it are v_dot2_f32_bf16 instructions on packed
+//            pairs (dequant_int4_word_bf16), which needs s/8 to be a normal bf16;
 //   general  (8u - 64) * (s/8) resp. (u - 128) * s: exact for every finite s, with the sign of
 //            a zero product as the reference's multiply gives it.
 // ---------------------------------------------------------------------------------------------
@@ -193,6 +194,10 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
+#ifndef MGEMV_BF16_DOT_DEQUANT
+#define MGEMV_BF16_DOT_DEQUANT 1
+#endif
+constexpr bool kBf16DotDequant = MGEMV_BF16_DOT_DEQUANT != 0;  // 0: the v_cvt / v_fma route for int4 as well
 constexpr int kActF16 = 0;
 constexpr int kActBf16 = 1;
 
@@ -206,13 +211,16 @@ __device__ __forceinline__ float byte_to_f32(uint32_t v) {
   return (float)((v >> (8 * BYTE)) & 0xffu);  // v_cvt_f32_ubyteN
 }
 
-// bf16 bit pattern of a scale for which the fused form is exact (both weight widths): 0x0001 .. 0x7aff.
-__device__ __forceinline__ bool fused_form_ok_bf16(uint32_t scale_bits) { return ((scale_bits & 0xffffu) - 1u) < 0x7affu; }
+// bf16 bit pattern of a scale for which the fused form is exact (both weight widths):
+// 0x0d80 .. 0x7aff, i.e. 2^-100 <= s < 2^119 -- positive, s/8 a normal bf16, -128 s finite.
+__device__ __forceinline__ bool fused_form_ok_bf16(uint32_t scale_bits) { return ((scale_bits & 0xffffu) - 0x0d80u) < (0x7b00u - 0x0d80u); }
 
 struct Bf16Scale {
-  float mul;  // int4: s/8; int8: s
-  float add;  // fused form: -8s resp. -128s; general form: unused
-  float z;    // additive zero
+  float mul;        // int4: s/8; int8: s
+  float add;        // fused form: -8s resp. -128s (int4 through the dot instructions: -24s); general form: unused
+  float z;          // additive zero
+  uint32_t sel_lo;  // int4 fused form through the dot instructions: the bf16 pairs (s/8, 0) ...
+  uint32_t sel_hi;  // ... and (0, s/8)
 };
 
 template <int BITS, bool FUSED>
@@ -220,8 +228,13 @@ __device__ __forceinline__ Bf16Scale make_bf16_scale(uint32_t s_bits, uint32_t z
   const float s = bf16_low_to_f32(s_bits);
   Bf16Scale f;
   f.mul = BITS == 4 ? s * 0.125f : s;
-  f.add = FUSED ? s * (BITS == 4 ? -8.0f : -128.0f) : 0.0f;
+  f.add = FUSED ? s * (BITS == 4 ? (kBf16DotDequant ? -24.0f : -8.0f) : -128.0f) : 0.0f;
   f.z = bf16_low_to_f32(z_bits);
+  f.sel_lo = f.sel_hi = 0;
+  if constexpr (BITS == 4 && FUSED && kBf16DotDequant) {
+    f.sel_lo = (s_bits & 0xffffu) - 0x0180u;  // s/8: three off the exponent of a normal s (the fused range has no other)
+    f.sel_hi = f.sel_lo << 16;
+  }
   return f;
 }
 
@@ -243,12 +256,60 @@ __device__ __forceinline__ uint32_t dequant_pair_bf16(float a, float b, const Bf
   return d;
 }
 
+// Eight bf16 values (four packed pairs a[0..3]) through out = rn_bf16(a * m + c), fp32 inside:
+// v_dot2_f32_bf16 with the factor pair sel_lo = (m, 0) resp. sel_hi = (0, m) computes
+// a.lo * m + c resp. a.hi * m + c straight from the packed pair -- fused, one rounding (checked
+// exhaustively by the tests) -- and v_cvt_pk_bf16_f32 rounds to bf16.  The product with the zero
+// factor vanishes as long as every a is finite, which the fused form's scale range guarantees.
+// One asm block, because the compiler does not know these are dot instructions: their results
+// must not be read by another kind of instruction within three issue slots, and the order
+// below keeps at least three instructions between each dot and the conversion that consumes it.
+__device__ __forceinline__ void dot_round_bf16x8(const uint32_t (&a)[4], uint32_t sel_lo, uint32_t sel_hi, float c,
+                                                 uint32_t (&out)[4]) {
+  float t0, t1, t2, t3, t4, t5, t6, t7;
+  asm("v_dot2_f32_bf16 %4, %12, %16, %18\n\t"
+      "v_dot2_f32_bf16 %5, %12, %17, %18\n\t"
+      "v_dot2_f32_bf16 %6, %13, %16, %18\n\t"
+      "v_dot2_f32_bf16 %7, %13, %17, %18\n\t"
+      "v_dot2_f32_bf16 %8, %14, %16, %18\n\t"
+      "v_dot2_f32_bf16 %9, %14, %17, %18\n\t"
+      "v_dot2_f32_bf16 %10, %15, %16, %18\n\t"
+      "v_dot2_f32_bf16 %11, %15, %17, %18\n\t"
+      "v_cvt_pk_bf16_f32 %0, %4, %5\n\t"
+      "v_cvt_pk_bf16_f32 %1, %6, %7\n\t"
+      "v_cvt_pk_bf16_f32 %2, %8, %9\n\t"
+      "v_cvt_pk_bf16_f32 %3, %10, %11"
+      : "=&v"(out[0]), "=&v"(out[1]), "=&v"(out[2]), "=&v"(out[3]), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3),
+        "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7)
+      : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(sel_lo), "v"(sel_hi), "v"(c));
+}
+
 // int4: the fields of elements (2,3) sit at bits 3-6 of bytes 0 and 2, those of (6,7) at bits 3-6
 // of bytes 1 and 3; (0,1) and (4,5) come to bytes 0 and 2 after a shift by 4 resp. a rotation
 // by 12 (tile_layout.h).  A masked byte converts to 8u.
 template <bool HAS_ZERO, bool FUSED>
 __device__ __forceinline__ void dequant_int4_word_bf16(uint32_t w, const ConvertRegs& c, const Bf16Scale& f,
                                                        uint32_t (&d)[4]) {
+  if constexpr (FUSED && kBf16DotDequant) {
+    // A field at bits 3-6 of a half-word under the bf16 pattern 0x4300 (128.0, mantissa step 1) IS
+    // the bf16 value 128 + 8u -- the route of gemv/interleaved_numeric_conversion.h:340-401 on
+    // these field positions -- and (128 + 8u) * (s/8) - 24 s = (u - 8) s exactly.
+    uint32_t magic;  // in a VGPR, so that mask (an SGPR) and magic fit one v_and_or_b32
+    asm("v_mov_b32 %0, 0x43004300" : "=v"(magic));
+    uint32_t m[4];
+    m[0] = ((w >> 4) & c.mask3) | magic;
+    m[1] = (w & c.mask3) | magic;
+    m[2] = (__builtin_amdgcn_alignbit(w, w, 12) & c.mask3) | magic;
+    m[3] = ((w >> 8) & c.mask3) | magic;
+    if constexpr (HAS_ZERO) {
+      uint32_t pb[4];
+      dot_round_bf16x8(m, f.sel_lo, f.sel_hi, f.add, pb);
+      dot_round_bf16x8(pb, 0x00003f80u, 0x3f800000u, f.z, d);   // factors (1, 0) and (0, 1)
+    } else {
+      dot_round_bf16x8(m, f.sel_lo, f.sel_hi, f.add, d);
+    }
+    return;
+  }
   const uint32_t e01 = (w >> 4) & c.mask3;
   const uint32_t e23 = w & c.mask3;
   const uint32_t e45 = __builtin_amdgcn_alignbit(w, w, 12) & c.mask3;

@@ -66,7 +66,7 @@ def test_dequant_every_finite_scale_bit_exact(gpu, bits, form):
     """Each (row, group) gets its own scale so that ALL finite bf16 scales (subnormals, huge values,
     both signs) meet every int4 weight value (a spread of int8 values), with an additive zero:
     multiply, round, add, round.  Consecutive bit patterns share a tile, so in "auto" the tiles
-    whose scales all lie in 0x0001..0x7aff take the fused form and the others the general one."""
+    whose scales all lie in 0x0d80..0x7aff take the fused form and the others the general one."""
     allbits = np.arange(65536, dtype=np.uint16)
     finite = allbits[(allbits & 0x7F80) != 0x7F80]            # 65280 values
     n_out, g = 64, 64
