@@ -1290,14 +1290,13 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
   }
   const int groups = ceil_div(tiles, tiles_per_wave);
-  // Measured on MI355X with the software-pipelined kernels (one tile group per workgroup is
-  // best throughout):
+  // Shapes that the exact-fit rule below does not take (measured on MI355X; one tile group per
+  // workgroup is best throughout):
   //  * about one workgroup per compute unit or fewer (<= 384 tile groups): few, longer waves --
   //    4 k-split waves, each pipelining two or more units -- beat more, shorter ones
-  //    (4096x4096: 4.37 us at 4 waves vs 4.57 us at 8);
-  //  * more tile groups than that: split as far as the units allow (at most 16 waves) while the
-  //    launch stays under ~8k waves, and fall back to two units per wave when that still
-  //    leaves >= 4096 waves (8192x8192: 10.6 us at 8 waves vs 11.2 us at 16).
+  //    (4096x4096: 4.08 us at 4 waves against 4.33 us at 8);
+  //  * more tile groups than that: split as far as the units allow while the launch stays under
+  //    ~8k waves, and fall back to two units per wave when that still leaves >= 4096 waves.
   const int max_waves = mc ? kMaxWavesPerMfmaWorkgroup
                         : m_batch >= 3 || knobs.wide_waves ? kMaxWavesPerWideWorkgroup
                                                   : kMaxWavesPerWorkgroup;

@@ -266,6 +266,39 @@ def test_tuned_plan_table_steers_exactly_its_problem(tmp_path):
         mg.set_launch_override(0, 0, 0, 0)
 
 
+def test_tuned_plan_table_is_safe_under_concurrent_writers_and_readers():
+    import threading
+    from mixed_gemv_amd import autotune
+    autotune.clear()
+    errors = []
+
+    def writer(t):
+        try:
+            for i in range(300):
+                mg.set_tuned_plan(64 * (1 + i % 50), 512 * (1 + t), 4, 128, 1, kernel=mg.KERNEL_VALU, split_k=1 + i % 4)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    def reader():
+        try:
+            for i in range(600):
+                q = mg.query_launch(64 * (1 + i % 50), 1, 512 * (1 + i % 4), 4, 128)
+                assert q["threads"] % 64 == 0 and q["workgroups"] >= 1
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=writer, args=(t,)) for t in range(4)] + [threading.Thread(target=reader) for _ in range(4)]
+    try:
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not errors, errors
+        assert mg.tuned_plan_count() == 4 * 50
+    finally:
+        autotune.clear()
+
+
 def test_adaptor_mirror_rejects_small_groups_like_the_reference():
     args = mg.GemvAdaptor.Arguments((64, 1, 512), 0x1000, 0x1000, 0x1000, 0x1000, None, 0x1000, group_size=32)
     with pytest.raises(MixedGemvError) as ei:
