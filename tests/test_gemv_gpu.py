@@ -469,6 +469,45 @@ def test_baseline_configs_full_size(gpu, cfg):
     check(prob, gpu, dequant=(mb == 1))
 
 
+def test_hip_graph_replays_match_eager_launches(gpu):
+    """The entry points neither allocate nor synchronise, so a caller may capture them; every replay of
+    a graph holding a VALU launch, both matrix-core launches and a bf16 launch must reproduce the eager
+    results bit for bit, with eager work and synchronisations between the replays."""
+    import torch
+    probs = [Problem("g_valu", 320, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=2, bias=True),
+             Problem("g_reg", 320, 2048, 4, SCALE_AND_ZEROS, 64, m_batch=6, bias=True),      # register-operand matrix core
+             Problem("g_lds", 320, 2048, 8, PER_COLUMN, 0, m_batch=16, bias=False),          # LDS-staged, 16 rows staged
+             Problem("g_bf16", 320, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True, element="bf16")]
+    devs = [DeviceProblem(p, gpu) for p in probs]
+    assert [mg.query_launch(320, p.m_batch, 2048, p.bits)["matrix_core"] for p in probs[:3]] == [0, 1, 2]
+    eager = [d.run().copy() for d in devs]
+
+    def launch_all():
+        for d in devs:
+            p = d.p
+            mg.device_gemv(d.w, d.x, d.scale, d.zero, d.bias, d.y, 1, p.n_out, p.m_batch, p.k, p.group_size,
+                           p.quant_op, p.bits, element=p.element)
+
+    launch_all()   # anything lazy (function attributes for large LDS) happens before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launch_all()
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(4):
+        for d in devs:
+            d.y.fill_(0x7e00)                     # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for d, want in zip(devs, eager):
+            got = d.y.cpu().numpy().view(want.dtype)
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (replay, d.p.tag)
+
+
 def test_reference_shipped_shape(gpu):
     """The shape the reference's main() ships with (mixed_gemv_test.cu:187-191), reduced 4x along
     the vocabulary dimension to keep the CPU side short: out = 37984, K = 2048, int4 g128 scale+zero."""
