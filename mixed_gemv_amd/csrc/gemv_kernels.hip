@@ -1528,9 +1528,23 @@ template <int BITS, int QOP, int GPR, int ROUNDS, int ACT>
 hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
   const auto kernel = gemv_mfma_lds_kernel<BITS, QOP, GPR, ROUNDS, ACT>;
   if (g.lds > 48 * 1024) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds);
-    if (e != hipSuccess) return e;
+    // More than 48 KiB of dynamic LDS has to be granted per kernel and device; remember the
+    // largest grant so that only the first such launch pays for the call.
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> granted[kMaxDevices];
+    static std::mutex grant_mutex;
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return hipErrorInvalidDevice;
+    const bool tracked = device >= 0 && device < kMaxDevices;
+    if (!tracked || granted[device].load() < (int)g.lds) {
+      std::lock_guard<std::mutex> lock(grant_mutex);  // grant and bookkeeping change together
+      if (!tracked || granted[device].load() < (int)g.lds) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds);
+        if (e != hipSuccess) return e;
+        if (tracked) granted[device].store((int)g.lds);
+      }
+    }
   }
   return launch(kernel, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale, g.zero_add, g.n_out, g.k,
                 pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups, g.tail.num_groups,
