@@ -641,20 +641,36 @@ __device__ __forceinline__ u32x4 mfma_operand(const LdsActivations<BITS>& xa, in
   return *reinterpret_cast<const u32x4*>(xa.lane_base + (i * G::kChunkK + j * 8) * 2);
 }
 
+// The activation operands of the matrix instructions of block i.
+template <int BITS, typename Activations>
+__device__ __forceinline__ void load_block_operands(const Activations& xa, int i, u32x4 (&ops)[BITS == 4 ? 4 : 2]) {
+#pragma unroll
+  for (int j = 0; j < (BITS == 4 ? 4 : 2); ++j) ops[j] = mfma_operand<BITS>(xa, i, j);
+}
+
 template <int BITS, int QOP, int GROUPS_PER_RUN, bool SHORT, int ACT, typename Activations>
 __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
                                                        const Activations& xa, const ConvertRegs& c,
                                                        half2_t col_scale2) {
   constexpr bool kHasZero = QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  constexpr int kFrags = BITS == 4 ? 4 : 2;
+  // The operands of block i+1 are requested before block i is dequantised, and the request is
+  // pinned there: left alone the compiler reads each operand right in front of its matrix
+  // instruction and the wave sits through the LDS latency sixteen times per unit.
+  u32x4 ops[2][kFrags];
+  load_block_operands<BITS>(xa, 0, ops[0]);
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i) {
+    if (i + 1 < kBlocksPerUnit) load_block_operands<BITS>(xa, i + 1, ops[(i + 1) & 1]);
+    __builtin_amdgcn_sched_barrier(0);
+    const u32x4 (&op)[kFrags] = ops[i & 1];
     const int gi = i * GROUPS_PER_RUN / kBlocksPerUnit;
     if constexpr (ACT == kActBf16) {
       // bf16: the same dequantiser as the VALU kernel (SHORT = fused form), v_mfma_f32_16x16x32_bf16
       const uint32_t s_bits = QOP != MGEMV_PER_COLUMN_SCALE_ONLY ? f.s[gi] : as_u32(col_scale2);
       const Bf16Scale bs = make_bf16_scale<BITS, SHORT>(s_bits, kHasZero ? f.z[gi] : 0u);
 #pragma unroll
-      for (int j = 0; j < (BITS == 4 ? 4 : 2); ++j) {
+      for (int j = 0; j < kFrags; ++j) {
         u32x4 a;
         if constexpr (BITS == 4) {
           uint32_t d[4];
@@ -667,7 +683,7 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
           a = u32x4{d0[0], d0[1], d1[0], d1[1]};
         }
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                      __builtin_bit_cast(bf16x8_t, mfma_operand<BITS>(xa, i, j)), acc, 0, 0, 0);
+                                                      __builtin_bit_cast(bf16x8_t, op[j]), acc, 0, 0, 0);
       }
       continue;
     }
@@ -692,7 +708,7 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
 #pragma unroll
         for (int h = 0; h < 4; ++h) a[h] = as_u32(d[h]);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
-                                                     __builtin_bit_cast(half8_t, mfma_operand<BITS>(xa, i, j)), acc, 0, 0, 0);
+                                                     __builtin_bit_cast(half8_t, op[j]), acc, 0, 0, 0);
       }
     } else {
 #pragma unroll
@@ -706,7 +722,7 @@ __device__ __forceinline__ void compute_unit_mfma_form(f32x4& acc, const MfmaWei
         a[2] = as_u32(dequant_pair<kHasZero>(q1[0], s2, z2));
         a[3] = as_u32(dequant_pair<kHasZero>(q1[1], s2, z2));
         acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a),
-                                                     __builtin_bit_cast(half8_t, mfma_operand<BITS>(xa, i, j)), acc, 0, 0, 0);
+                                                     __builtin_bit_cast(half8_t, op[j]), acc, 0, 0, 0);
       }
     }
   }
