@@ -1,4 +1,5 @@
 """Builds the HIP library in-tree: mixed_gemv_amd/lib/libmixed_gemv_amd.so (gfx950 only)."""
+import concurrent.futures
 import os
 import shutil
 import subprocess
@@ -10,7 +11,8 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmixed_gemv_amd.so")
 
-SOURCES = ["gemv_kernels.hip", "host_utils.cpp"]
+# One translation unit per family of kernel instantiations, so that they compile side by side.
+SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "gemv_kernels.hip", "host_utils.cpp"]
 
 # -ffp-contract=off: the dequantiser is a separately rounded fp16 multiply and add.
 # -packed-fp32-ops off: keep the compiler from forming v_pk_*_f32.
@@ -32,17 +34,21 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build_library(verbose=True, extra_flags=()):
+def build_library(verbose=True, extra_flags=(), jobs=None):
     os.makedirs(LIB_DIR, exist_ok=True)
-    objs = []
-    for src in SOURCES:
+    jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
+
+    def compile_one(src):
         obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
         cmd = [hipcc(), *HIP_FLAGS, *extra_flags, "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC,
                "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)
-        objs.append(obj)
+        return obj
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fopenmp", *objs, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)

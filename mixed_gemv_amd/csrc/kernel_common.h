@@ -1,0 +1,167 @@
+// Shared by the kernels of this library and their launchers: launch constants, the kernel
+// argument block, small device helpers, and the host-side description of a launch.
+#ifndef MIXED_GEMV_AMD_KERNEL_COMMON_H_
+#define MIXED_GEMV_AMD_KERNEL_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include "device_math.h"
+#include "mixed_gemv.h"
+#include "tile_layout.h"
+
+namespace mgemv {
+
+constexpr int kWave = 64;
+constexpr int kMaxWavesPerWorkgroup = 16;
+constexpr int kMaxWavesPerWideWorkgroup = 8;  // VALU kernel with 3-4 activation rows: 256 VGPRs per wave
+constexpr int kMaxWavesPerMfmaWorkgroup = 8;  // leaves each wave of the matrix-core kernel 256 VGPRs
+constexpr int kNumXcd = 8;
+constexpr int kNumCus = 256;
+constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
+constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
+
+// Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are what a
+// wave needs to address its first loads, and they are preloaded into SGPRs (build flag
+// -amdgpu-kernarg-preload-count=14); everything else sits in GemvTail.
+struct GemvTail {
+  const half_t* bias;
+  half_t* y;
+  int split_k;         // waves of a workgroup that share one tile (blockDim.x / 64)
+  int m_batch;         // activation rows (matrix-core kernel)
+  int num_groups;      // k / group_size (1 in per-column mode): extent of the scale / zero tables
+  int flags;           // kExactIntegerFormOnly or 0
+  int seq_base;        // VALU kernel: tiles / sequences ...
+  int seq_rem;         // ... and tiles % sequences (the first seq_rem sequences get one tile more)
+  long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
+};
+
+// Scalar view of one problem inside a kernel.
+struct Problem {
+  const uint8_t* weights;
+  const half_t* x;
+  const half_t* scale;
+  const half_t* zero_add;
+  int n_out;
+  int k;
+  int ksteps;          // ceil(k / kStepK)
+  int steps_per_wave;  // units per wave
+  int workgroups;      // logical workgroups = ceil(tiles / tiles_per_wg)
+  int wgs_per_xcd;     // ceil(workgroups / 8); gridDim.x = 8 * wgs_per_xcd
+  int group_size;
+  int tiles_per_wg;    // blockDim.y
+};
+
+constexpr uint32_t pack_steps(int ksteps, int steps_per_wave) { return (uint32_t)ksteps | ((uint32_t)steps_per_wave << 16); }
+constexpr uint32_t pack_group(int group_size, int tiles_per_wg) { return (uint32_t)group_size | ((uint32_t)tiles_per_wg << 24); }
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Neighbouring tiles read
+// neighbouring 32-byte pieces of the same scale/zero cache lines, so give each XCD (and its
+// private L2) a contiguous range of tiles instead of every eighth one.
+__device__ __forceinline__ int logical_workgroup(const Problem& p) {
+  const int xcd = blockIdx.x % kNumXcd;
+  const int slot = blockIdx.x / kNumXcd;
+  return xcd * p.wgs_per_xcd + slot;
+}
+
+// Group index of reduction position k_index (host/mixed_gemv.h:88), clamped to the last
+// group for the padded positions past k.
+__device__ __forceinline__ int group_of(const Problem& p, int k_index) {
+  k_index = k_index < p.k ? k_index : p.k - 1;
+  const bool pow2 = (p.group_size & (p.group_size - 1)) == 0;
+  return pow2 ? (k_index >> __builtin_ctz((unsigned)p.group_size)) : (k_index / p.group_size);
+}
+
+// 16-bit buffer load into the low half of a 32-bit register.  The upper half is left
+// unspecified on purpose: zero-extending it would be a VALU instruction on the loaded value,
+// and the compiler places that instruction -- and the wait for the data -- next to the load,
+// in front of the loads that should be issued behind it.
+__device__ __forceinline__ uint32_t load_b16_low(__amdgpu_buffer_rsrc_t rsrc, int voffset) {
+  const uint16_t bits = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, voffset, 0, kCacheDefault);
+  half2_t v;  // element 1 deliberately not set
+  v[0] = __builtin_bit_cast(half_t, bits);
+  return as_u32(v);
+}
+__device__ __forceinline__ uint32_t load_half_bits(const half_t* p) {
+  return (uint32_t)*reinterpret_cast<const uint16_t*>(p);
+}
+__device__ __forceinline__ half2_t splat_low(uint32_t bits) {
+  const half_t h = __builtin_bit_cast(half_t, (uint16_t)bits);
+  return half2_t{h, h};
+}
+
+struct ScaleTables {
+  __amdgpu_buffer_rsrc_t scale, zero;
+};
+
+// True when the scale of every lane of the wave (all groups of the unit) permits the short
+// (fp16, int4) resp. fused (bf16) dequantiser; wave-uniform, so the choice costs one scalar
+// branch per unit.
+template <int ACT, typename Bits, int GROUPS_PER_RUN>
+__device__ __forceinline__ bool wave_scales_permit_short_form(const Bits (&scale_bits)[GROUPS_PER_RUN]) {
+  bool ok = true;
+#pragma unroll
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi)
+    ok = ok && (ACT == kActBf16 ? fused_form_ok_bf16(scale_bits[gi]) : short_form_ok(scale_bits[gi]));
+  return __builtin_amdgcn_ballot_w64(!ok) == 0;
+}
+
+// Sum over the four k slices of a wave: lanes l, l+16, l+32, l+48 hold the same row.
+// The result is valid in lanes 0..15.
+__device__ __forceinline__ float reduce_k_slices(float v) {
+  v += __shfl_down(v, 32);
+  v += __shfl_down(v, 16);
+  return v;
+}
+
+// The lane number, recomputed.  Used behind the unit loop so that the value computed in front
+// of it need not stay in a register (or be spilled) across the loop.
+__device__ __forceinline__ int lane_after_loop() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------------------------
+
+struct LaunchPlan {
+  int split_k, tiles_per_wg, steps_per_wave, workgroups, wgs_per_xcd, threads;
+  int tiles_per_wave;  // 1 on the VALU path; 1, 2 or 4 on the matrix-core path
+  int tiles_in_sequence;  // VALU path: most tiles any wave walks one after the other
+  int staged_rows;        // LDS-staged matrix-core kernel: 8 or 16 activation rows per stage; 0 = other kernels
+  bool matrix_core;       // one of the two matrix-core kernels (else the VALU kernel)
+};
+
+// Launches through hipLaunchKernel so that the status returned is this launch's own, not a
+// stale sticky error left behind by some other runtime call of the process.
+template <typename Kernel, typename... Args>
+hipError_t launch(Kernel kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+  void* argv[] = {static_cast<void*>(&args)...};
+  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, argv, lds, stream);
+}
+
+// Host-side description of one GEMV launch.
+struct GemvLaunch {
+  const uint8_t* weights;
+  const half_t* x;
+  const half_t* scale;
+  const half_t* zero_add;
+  int n_out, k, group_size;
+  LaunchPlan plan;
+  GemvTail tail;
+  dim3 grid, block;
+  size_t lds;
+  hipStream_t stream;
+};
+
+// Dispatchers, one translation unit each (the kernels are templates on weight width, quant mode,
+// activation rows, groups per run, ...; the run-time values pick the instantiation).
+hipError_t launch_gemv_f16(const GemvLaunch& g, int bits, int qop, int mb, int gpr);
+hipError_t launch_gemv_bf16(const GemvLaunch& g, int bits, int qop, int mb, int gpr);
+hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr);
+hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act);
+
+}  // namespace mgemv
+
+#endif  // MIXED_GEMV_AMD_KERNEL_COMMON_H_

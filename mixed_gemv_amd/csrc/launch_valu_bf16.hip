@@ -1,0 +1,10 @@
+// bfloat16 instantiations of the VALU GEMV kernel.
+#include "gemv_dpp_kernel.h"
+
+namespace mgemv {
+
+hipError_t launch_gemv_bf16(const GemvLaunch& g, int bits, int qop, int mb, int gpr) {
+  return launch_gemv_act<kActBf16>(g, bits, qop, mb, gpr);
+}
+
+}  // namespace mgemv
