@@ -1,18 +1,6 @@
 // C-ABI entry points of the device side: argument checks, launch geometry, tuned plans, and the
 // dequantise kernel.  The GEMV kernels live in gemv_dpp_kernel.h (VALU) and launch_mfma.hip
 // (matrix cores).
-//
-// One wavefront works on a contiguous range of k steps (units of tile_layout.h) of one 16-row
-// tile of the weight matrix, or of several consecutive tiles one after the other.  Per unit it
-// issues four 1-KiB weight loads, one activation load and the scale/zero loads, dequantises
-// in packed fp16 to the bits of gemv/warp/warp_dequantizer.h:52-59 (rounded product, then
-// rounded sum), and accumulates in fp32 with v_dot2c_f32_f16 whose activation operand is a DPP
-// row broadcast.  Several waves of a workgroup split the k range of the same tiles (split-K);
-// their per-lane partial sums meet in LDS, are summed in a fixed order, biased, rounded to
-// fp16 and stored.  This covers, for the reference, the main loops
-// of gemv/threadblock/dq_mma_singlestage_{finegrained,percol}.h, the reductions of
-// gemv/warp/reduce.h and gemv/threadblock/accumulator_combine.h, and the epilogue of
-// epilogue/threadblock/epilogue.h.
 #include <hip/hip_runtime.h>
 
 #include <atomic>
