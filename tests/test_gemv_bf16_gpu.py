@@ -46,6 +46,8 @@ SMALL = [
     ("b_i4_tiny", 4, 64, 4, SCALE_AND_ZEROS, 64, 1, True),
     ("b_i4_mb7", 64, 1024, 4, SCALE_AND_ZEROS, 64, 7, False),       # two launches of the VALU kernel
     ("b_i8_mb16", 48, 512, 8, PER_COLUMN, 0, 16, True),
+    ("b_i4_one_tile_mb7", 16, 512, 4, SCALE_AND_ZEROS, 128, 7, True),   # a single tile: no matrix-core kernel fits
+    ("b_i4_two_tiles_mb12", 20, 1024, 4, SCALE_AND_ZEROS, 128, 12, False),
 ]
 
 

@@ -51,6 +51,8 @@ SMALL = [
     ("s_i4_mb7", 64, 1024, 4, SCALE_AND_ZEROS, 64, 7, False),
     ("s_i4_mb16", 48, 1024, 4, SCALE_AND_ZEROS, 128, 16, True),
     ("s_i8_mb9", 48, 512, 8, PER_COLUMN, 0, 9, True),
+    ("s_i4_one_tile_mb7", 16, 512, 4, SCALE_AND_ZEROS, 128, 7, True),   # a single tile: register-operand matrix core
+    ("s_i4_two_tiles_mb12", 20, 1024, 4, SCALE_AND_ZEROS, 128, 12, False),
 ]
 
 
