@@ -150,13 +150,14 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
   return it == g_tuned_plans.end() ? kn : it->second;
 }
 
-// Built-in rule, measured: up to 4 activation rows the VALU kernel wins on matrices of up to
-// ~8k units (8192x8192: 12.0 us at 4 rows against 11.8 us, 10.9 against 11.9 at 3); on larger ones
-// the LDS-staged matrix-core kernel already wins at 3 rows (28672x8192: 26.9 us against 31.9 us).
+// Built-in rule, measured (VALU kernel against the matrix-core kernel the plan would pick, us):
+//   4096x4096 (2 k units):   4 rows 5.2 / 5.5,   5 rows 8.8 / 5.5
+//   8192x8192 (8 k units):   3 rows 10.8 / 11.2, 4 rows 11.8 / 11.2
+//   28672x8192 (28 k units): 2 rows 27.5 / 26.2, 3 rows 31.9 / 26.7
 // From 5 rows the VALU kernel would need a second launch.
 inline bool use_matrix_cores(int m_batch, long long units, int forced) {
   if (forced > 0) return m_batch >= forced;
-  return m_batch >= 5 || (m_batch >= 3 && units >= 16384);
+  return m_batch >= 5 || (m_batch >= 4 && units >= 8192) || (m_batch >= 3 && units >= 16384);
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
