@@ -1,12 +1,13 @@
 #!/usr/bin/env python3
-"""Writes tests/golden/gemv_cases.npz: small seeded problems with their expected dequantised
-weights and outputs.
+"""Writes tests/golden/gemv_cases.npz and gemv_cases_bf16.npz: small seeded problems with their
+expected dequantised weights and outputs (fp16 and bfloat16 elements).
 
 The reference ships no vectors of its own (its only test draws from std::random_device and
 prints differences), and its host code cannot be compiled here (it needs NVIDIA CUTLASS
 v3.4.1 and CUDA headers), so the expected values are produced by the C oracle and, before
 they are written, required to be bit-identical to the independent numpy restatement in
-tests/np_restate.py.  The file pins both against silent drift.
+tests/np_restate.py (fp16) or the torch.bfloat16 restatement in tests/torch_restate.py (bf16).
+The files pin both against silent drift.
 
 Run from the repository root:  python tests/golden/make_golden.py
 """
@@ -34,9 +35,40 @@ CASES = [
 ]
 
 
-def build(case):
+def build(case, element="f16"):
     tag, n, k, bits, qop, g, mb, bias, zk, xd = case
-    return Problem(tag, n, k, bits, qop, g, m_batch=mb, bias=bias, zero_kind=zk, x_dist=xd)
+    return Problem(tag, n, k, bits, qop, g, m_batch=mb, bias=bias, zero_kind=zk, x_dist=xd, element=element)
+
+
+def main_bf16():
+    import torch
+    import torch_restate
+    out = {}
+    for case in CASES:
+        tag = "b" + case[0][1:]
+        p = build((tag,) + case[1:], element="bf16")
+        dq = p.oracle_dequant()
+        y = p.oracle_gemv(threads=1)
+        q = p.q.reshape(p.n_out, p.k).astype(np.int32)
+        ref_dq = torch_restate.torch_dequantize(q, p.scale, p.zero_add, p.group_size)
+        ref_y = torch_restate.sequential_gemv(ref_dq, p.x, p.bias)
+        assert np.array_equal(dq, ref_dq.view(torch.int16).numpy().view(np.uint16)), tag
+        assert np.array_equal(y, ref_y), tag
+        out[f"{tag}/w_raw"] = p.w_raw
+        out[f"{tag}/x"] = p.x
+        out[f"{tag}/scale"] = p.scale
+        if p.zero_add is not None:
+            out[f"{tag}/zero_add"] = p.zero_add
+        if p.zeros_i8 is not None:
+            out[f"{tag}/zeros_i8"] = p.zeros_i8
+        if p.bias is not None:
+            out[f"{tag}/bias"] = p.bias
+        out[f"{tag}/dequant"] = dq
+        out[f"{tag}/y"] = y
+        out[f"{tag}/meta"] = np.array([p.n_out, p.k, p.bits, p.quant_op, p.group_size, p.m_batch], dtype=np.int64)
+    path = os.path.join(HERE, "gemv_cases_bf16.npz")
+    np.savez_compressed(path, **out)
+    print("wrote", path, os.path.getsize(path), "bytes")
 
 
 def main():
@@ -70,3 +102,4 @@ def main():
 
 if __name__ == "__main__":
     main()
+    main_bf16()
