@@ -37,8 +37,9 @@ def candidate_plans(n_out, k, weight_bits, m_batch):
                 out.append(dict(kernel=api.KERNEL_VALU, split_k=split_k, tiles_per_wg=tiles_per_wg,
                                 max_workgroups=cap))
     if m_batch >= 2:
-        for split_k in (1, 2, 4):
-            out.append(dict(kernel=api.KERNEL_MATRIX_CORE_LDS_STAGED, split_k=split_k))
+        for tiles_per_wg in (1, 2, 4):   # 1 or 2 tiles share 8 staged rows, 2 or 4 share 16; others fall back to 2
+            for split_k in (1, 2, 4):
+                out.append(dict(kernel=api.KERNEL_MATRIX_CORE_LDS_STAGED, split_k=split_k, tiles_per_wg=tiles_per_wg))
         for tiles_per_wave in (1, 2):
             for split_k in (2, 4, 8):
                 out.append(dict(kernel=api.KERNEL_MATRIX_CORE_REGISTER_OPERAND, split_k=split_k,

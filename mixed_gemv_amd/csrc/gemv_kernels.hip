@@ -167,11 +167,14 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
   const bool mc = use_matrix_cores(m_batch, (long long)tiles * ksteps, knobs.matrix_core_min_batch);
-  // Up to 256 tiles and 8 rows the register-operand kernel with one tile per wave wins: a lane of
-  // a row past m_batch loads nothing there, and no barrier ties the waves of a workgroup together
-  // (1024x2048, 5 rows: 3.6 us against 4.6 us; 4096x11008: 10.2 against 13.3; 4096x4096, 8 rows: 6.3
-  // against 6.7; at 16 rows, or from 384 tiles, the LDS-staged kernel is level or ahead).
-  const bool small_problem = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && tiles <= 256 && m_batch <= 8;
+  // Small problems (up to 256 tiles) with few rows or a short reduction take the register-operand
+  // kernel with one tile per wave: a lane of a row past m_batch loads nothing there, and no barrier
+  // ties the waves of a workgroup together (1024x2048, 5 rows: 3.4 us against 4.6 us LDS-staged;
+  // 4096x11008, 5 rows: 10.1 against 13.3; 1024x2048, 16 rows: 4.4 against 4.9).  From 7 rows the
+  // LDS-staged kernel with one tile per workgroup is ahead again (4096x4096, 8 rows: 5.4 against
+  // 6.1; 2048x8192: 7.5 against 8.9), and so it is from 384 tiles at any row count.
+  const bool small_problem = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && tiles <= 256 &&
+                             (m_batch <= 6 || ksteps <= 4);
   if (mc && knobs.matrix_core_variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND && !small_problem && tiles >= 2) {
     // LDS-staged kernel: two tiles per workgroup share the activation stage; k split as long as
     // the launch stays within 2048 waves (measured: 8192x8192 best at 4 k-split waves, 11008x4096
@@ -179,12 +182,21 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // workgroup per compute unit for 344 workgroups --, 28672x8192 at 1).
     LaunchPlan lp{};
     lp.matrix_core = true;
-    lp.tiles_per_wg = 2;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
+    // Tiles per workgroup = waves that share one activation stage.  Measured: one tile (8 staged
+    // rows) on small matrices, where two would leave compute units idle (4096x4096, 8 rows: 5.4 us
+    // against 6.4); four tiles (16 staged rows) on large ones, where the stage traffic matters
+    // (11008x4096, 16 rows: 10.1 against 11.3; 28672x8192: 30.2 against 32.8; 8192x8192 with its
+    // 512 tiles still prefers two: 13.5 against 17.7).
+    lp.tiles_per_wg = lp.staged_rows == 8 ? (tiles <= 256 ? 1 : 2) : (tiles >= 640 ? 4 : 2);
+    // the kernel exists for 4 or 8 staged rows per wave of a k range: 1 or 2 tiles share 8 rows, 2 or 4 share 16
+    if (ov_tw > 0 && (lp.staged_rows / ov_tw == 4 || lp.staged_rows / ov_tw == 8) && lp.staged_rows % ov_tw == 0)
+      lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
+    const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;
-    while (split < 4 && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 2048) split *= 2;
-    if (ov_sk > 0) split = ov_sk > 4 ? 4 : ov_sk;
+    while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 2048) split *= 2;
+    if (ov_sk > 0) split = ov_sk > max_split ? max_split : ov_sk;
     if (split > ksteps) split = ksteps;
     lp.steps_per_wave = ceil_div(ksteps, split);
     lp.split_k = ceil_div(ksteps, lp.steps_per_wave);
