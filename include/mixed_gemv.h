@@ -180,7 +180,7 @@ MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Which of the two matrix-core kernels serves the small batches:
  *   MGEMV_MATRIX_CORE_AUTO (default)          the register-operand kernel, one tile per wave, on matrices
- *                                             of up to 256 16-row tiles with up to 6 activation rows or
+ *                                             of up to 256 16-row tiles with up to 5 activation rows or
  *                                             a reduction of up to 4 k steps, else the LDS-staged kernel;
  *   MGEMV_MATRIX_CORE_REGISTER_OPERAND        always the kernel that reads its activation operand from
  *                                             L2 into registers;

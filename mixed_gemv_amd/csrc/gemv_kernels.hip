@@ -170,28 +170,30 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   // Small problems (up to 256 tiles) with few rows or a short reduction take the register-operand
   // kernel with one tile per wave: a lane of a row past m_batch loads nothing there, and no barrier
   // ties the waves of a workgroup together (1024x2048, 5 rows: 3.4 us against 4.6 us LDS-staged;
-  // 4096x11008, 5 rows: 10.1 against 13.3; 1024x2048, 16 rows: 4.4 against 4.9).  From 7 rows the
-  // LDS-staged kernel with one tile per workgroup is ahead again (4096x4096, 8 rows: 5.4 against
-  // 6.1; 2048x8192: 7.5 against 8.9), and so it is from 384 tiles at any row count.
+  // 2048x2048, 6 rows: 3.7 against 3.8; 1024x2048, 16 rows: 4.4 against 4.9).  With a longer
+  // reduction the LDS-staged kernel with one tile per workgroup is level at 5 rows and ahead from 6
+  // (4096x4096: 5.4 against 5.6 at 6 rows, 5.4 against 6.1 at 8; 2048x8192, 6 rows: 7.5 against 7.9),
+  // and so it is from 384 tiles at any row count.
   const bool small_problem = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && tiles <= 256 &&
-                             (m_batch <= 6 || ksteps <= 4);
+                             (m_batch <= 5 || ksteps <= 4);
   if (mc && knobs.matrix_core_variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND && !small_problem && tiles >= 2) {
-    // LDS-staged kernel: two tiles per workgroup share the activation stage; k split as long as
+    // LDS-staged kernel: the tiles of a workgroup share the activation stage; k split as long as
     // the launch stays within 2048 waves (measured: 8192x8192 best at 4 k-split waves, 11008x4096
-    // at 2 -- 11.4 us against 14.2 us at 4 with 16 rows, whose 133 KB of stages would leave one
-    // workgroup per compute unit for 344 workgroups --, 28672x8192 at 1).
+    // at 2, 28672x8192 at 1).
     LaunchPlan lp{};
     lp.matrix_core = true;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
-    // Tiles per workgroup = waves that share one activation stage.  Measured: one tile (8 staged
-    // rows) on small matrices, where two would leave compute units idle (4096x4096, 8 rows: 5.4 us
-    // against 6.4); four tiles (16 staged rows) on large ones, where the stage traffic matters
-    // (11008x4096, 16 rows: 10.1 against 11.3; 28672x8192: 30.2 against 32.8; 8192x8192 with its
-    // 512 tiles still prefers two: 13.5 against 17.7).
-    lp.tiles_per_wg = lp.staged_rows == 8 ? (tiles <= 256 ? 1 : 2) : (tiles >= 640 ? 4 : 2);
-    // the kernel exists for 4 or 8 staged rows per wave of a k range: 1 or 2 tiles share 8 rows, 2 or 4 share 16
-    if (ov_tw > 0 && (lp.staged_rows / ov_tw == 4 || lp.staged_rows / ov_tw == 8) && lp.staged_rows % ov_tw == 0)
-      lp.tiles_per_wg = ov_tw;
+    // Tiles per workgroup = waves that share one activation stage: as many as still leave about
+    // 170 workgroups (two thirds of the compute units), at most 8 and at most half the staged rows.
+    // Measured, 16 rows: 4096x4096 (256 tiles) 6.3 us at 1 tile against 7.2 at 2; 8192x8192 (512)
+    // 13.4 at 2 against 17.8 at 4; 11008x4096 (688) 10.1 at 4 against 11.3 at 2 and 14.2 at 8;
+    // 28672x8192 (1792) 28.3 at 8 against 30.6 at 4 and 32.8 at 2.  8 rows: 4096x4096 5.4 at 1
+    // against 6.4 at 2; 11008x4096 9.0 at 4 against 9.7 at 2; 28672x8192 27.6 at 4 against 29.5 at 2.
+    lp.tiles_per_wg = 1;
+    for (int tw = 2; tw <= 8 && tw * 2 <= lp.staged_rows; tw *= 2)
+      if (ceil_div(tiles, tw) >= 170) lp.tiles_per_wg = tw;
+    // the kernel exists for 2, 4, 8 or 16 staged rows per wave of a k range
+    if (ov_tw > 0 && ov_tw <= 8 && lp.staged_rows % ov_tw == 0 && lp.staged_rows / ov_tw >= 2) lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
     const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;

@@ -630,8 +630,12 @@ hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
 
 template <int BITS, int QOP, int GPR, int ACT>
 hipError_t launch_mfma_lds_kernel(const GemvLaunch& g, int rounds) {
-  return rounds == 4 ? launch_mfma_lds_kernel_r<BITS, QOP, GPR, 4, ACT>(g)
-                     : launch_mfma_lds_kernel_r<BITS, QOP, GPR, 8, ACT>(g);
+  switch (rounds) {
+    case 2: return launch_mfma_lds_kernel_r<BITS, QOP, GPR, 2, ACT>(g);
+    case 4: return launch_mfma_lds_kernel_r<BITS, QOP, GPR, 4, ACT>(g);
+    case 8: return launch_mfma_lds_kernel_r<BITS, QOP, GPR, 8, ACT>(g);
+    default: return launch_mfma_lds_kernel_r<BITS, QOP, GPR, 16, ACT>(g);
+  }
 }
 
 template <int BITS, int QOP, int ACT>

@@ -333,7 +333,7 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     y_all = dev.run().copy()
     assert np.array_equal(y_all.view(np.uint16), dev.run().view(np.uint16))
     assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (0 if m_batch < 5 else 1)   # few tiles, short k: register operand
-    assert mg.query_launch(80, m_batch, 4096, 4)["matrix_core"] == (0 if m_batch < 5 else 1 if m_batch <= 6 else 2)
+    assert mg.query_launch(80, m_batch, 4096, 4)["matrix_core"] == (0 if m_batch < 5 else 1 if m_batch <= 5 else 2)
     assert mg.query_launch(80, 7, 2048, 4)["matrix_core"] == 1   # few tiles, <= 8 rows: register operand
     assert mg.query_launch(8192, 7, 2048, 4)["matrix_core"] == 2
     single = Problem("rows", 80, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True)
