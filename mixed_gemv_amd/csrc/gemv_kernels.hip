@@ -157,7 +157,8 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 // From 5 rows the VALU kernel would need a second launch.
 inline bool use_matrix_cores(int m_batch, long long units, int forced) {
   if (forced > 0) return m_batch >= forced;
-  return m_batch >= 5 || (m_batch >= 4 && units >= 8192) || (m_batch >= 3 && units >= 16384);
+  return m_batch >= 5 || (m_batch >= 4 && units >= 8192) || (m_batch >= 3 && units >= 16384) ||
+         (m_batch >= 2 && units >= 24576);
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
