@@ -247,8 +247,11 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // of four waves per compute unit -- one wave per SIMD, all with the same amount of work --
     // beats any over-subscribed launch (8192x8192: 8.7 us against 10.2 us; 28672x8192: 2 %).
     // The four waves are tw tile sequences x 4/tw k-split waves, tw as large as still fits evenly.
+    // Walks of more than 7 tiles lose to one tile per workgroup (128256x4096, 8 tiles per wave:
+    // 51.5 us against 47.3; 151936x2048, 19 tiles: 31.9 against 29.8), so those are left out.
     for (int tw = 4; tw >= 1; tw /= 2) {
       const int sequences = kNumCus * tw;
+      if (ceil_div(tiles, sequences) > 7) continue;
       if ((long long)ceil_div(tiles, sequences) * sequences * 100 <= (long long)tiles * 103) {
         tiles_per_wg = tw;
         split_k = 4 / tw;

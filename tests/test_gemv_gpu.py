@@ -450,7 +450,7 @@ FULL = [
 FIT = [
     ("fit_tw4_two_tiles_each", 32032, 2048, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
     ("fit_tw2_long_k", 8192, 28672, 4, SCALE_AND_ZEROS, 128, 1, True, "normal", (0.001, 0.02)),
-    ("fit_vocab", 128256, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
+    ("fit_tw1_seven_tiles", 28672, 2048, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
     ("fit_int8_tw2", 8192, 4096, 8, PER_COLUMN, 0, 2, True, "uniform", (0.001, 0.01)),
 ]
 
@@ -461,6 +461,15 @@ def test_exact_fit_launches_full_size(gpu, cfg):
     plan = mg.query_launch(n_out, mb, k, bits)
     assert plan["workgroups"] == 256 and plan["threads"] == 256, plan
     prob = Problem(tag, n_out, k, bits, qop, g, m_batch=mb, bias=bias, x_dist=xd, scale_range=sr)
+    check(prob, gpu, dequant=False)
+
+
+def test_vocabulary_projection_one_tile_per_workgroup(gpu):
+    """128256 x 4096 (8016 tiles): an exact fit would mean walks of 8 tiles, which measured slower than one
+    tile per workgroup, so this shape launches one single-wave workgroup per tile."""
+    plan = mg.query_launch(128256, 1, 4096, 4)
+    assert plan["tiles_in_sequence"] == 1 and plan["workgroups"] == 8016, plan
+    prob = Problem("vocab", 128256, 4096, 4, SCALE_AND_ZEROS, 128, x_dist="normal")
     check(prob, gpu, dequant=False)
 
 
