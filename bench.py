@@ -42,6 +42,9 @@ WORKLOADS = {
            "int4 group-64 scale+zero GEMV + bias, N=K=8192"),
     "c5": (28672, 8192, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
            "int4 group-128 scale+zero GEMV, M=1, K=8192, N=28672"),
+    # not a BASELINE config: a vocabulary projection, the longest launch a decoder step has
+    "vocab": (128256, 4096, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
+              "int4 group-128 scale+zero GEMV, M=1, K=4096, N=128256 (vocabulary projection)"),
 }
 
 
@@ -335,7 +338,7 @@ def main():
     ap.add_argument("--launch", default="graph", choices=["graph", "stream"],
                     help="graph: the steps are replayed from a captured HIP graph (one kernel node per step, one "
                          "rotation of the buffer sets per replay); stream: one host launch per step")
-    ap.add_argument("--extra", default="c5,nsx8,nsx16,ns:bf16,c5:bf16",
+    ap.add_argument("--extra", default="c5,vocab,nsx8,nsx16,ns:bf16,c5:bf16",
                     help="comma list of further workloads reported under 'other_workloads' ('' = none); "
                          "'<name>x<B>' runs B problems per launch through the batched entry point, "
                          "'<name>:bf16' runs the bfloat16 entry point")
