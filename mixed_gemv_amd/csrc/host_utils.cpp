@@ -72,64 +72,92 @@ int bits_of_quant_type(int quant_type) {
 // low nibble = even index).  Blocked so that both sides are walked in cache-sized tiles.
 void transpose_quantised(uint8_t* dst, const uint8_t* src, size_t k, size_t n_out, int bits) {
   constexpr size_t kBlock = 64;
-  if (bits == 8) {
-    for (size_t k0 = 0; k0 < k; k0 += kBlock)
-      for (size_t n0 = 0; n0 < n_out; n0 += kBlock) {
-        const size_t k1 = k0 + kBlock < k ? k0 + kBlock : k;
-        const size_t n1 = n0 + kBlock < n_out ? n0 + kBlock : n_out;
+  const long long n_blocks = (long long)((n_out + kBlock - 1) / kBlock);
+  // one thread per block of 64 output rows: no two threads write the same byte (k is even)
+#pragma omp parallel for schedule(static)
+  for (long long nb = 0; nb < n_blocks; ++nb) {
+    const size_t n0 = (size_t)nb * kBlock;
+    const size_t n1 = n0 + kBlock < n_out ? n0 + kBlock : n_out;
+    if (bits == 4) std::memset(dst + n0 * k / 2, 0, (n1 - n0) * k / 2);
+    for (size_t k0 = 0; k0 < k; k0 += kBlock) {
+      const size_t k1 = k0 + kBlock < k ? k0 + kBlock : k;
+      if (bits == 8) {
         for (size_t n = n0; n < n1; ++n)
           for (size_t kk = k0; kk < k1; ++kk) dst[n * k + kk] = src[kk * n_out + n];
+      } else {
+        for (size_t n = n0; n < n1; ++n)
+          for (size_t kk = k0; kk < k1; ++kk) {
+            const size_t si = kk * n_out + n;
+            const uint8_t v = (uint8_t)((src[si >> 1] >> (4 * (si & 1))) & 0xfu);
+            const size_t di = n * k + kk;
+            dst[di >> 1] = (uint8_t)(dst[di >> 1] | (v << (4 * (di & 1))));
+          }
       }
-    return;
-  }
-  std::memset(dst, 0, n_out * k / 2);
-  for (size_t k0 = 0; k0 < k; k0 += kBlock)
-    for (size_t n0 = 0; n0 < n_out; n0 += kBlock) {
-      const size_t k1 = k0 + kBlock < k ? k0 + kBlock : k;
-      const size_t n1 = n0 + kBlock < n_out ? n0 + kBlock : n_out;
-      for (size_t n = n0; n < n1; ++n)
-        for (size_t kk = k0; kk < k1; ++kk) {
-          const size_t si = kk * n_out + n;
-          const uint8_t v = (uint8_t)((src[si >> 1] >> (4 * (si & 1))) & 0xfu);
-          const size_t di = n * k + kk;
-          dst[di >> 1] = (uint8_t)(dst[di >> 1] | (v << (4 * (di & 1))));
-        }
     }
+  }
+}
+
+// Walks the chunks of row n in ascending k and hands each (source byte offset inside the row,
+// byte offset inside the tiled buffer) to `visit`; nested loops instead of chunk_offset() keep
+// integer divisions out of the inner loop.
+template <typename Visit>
+inline void for_each_chunk_of_row(size_t n, size_t k, size_t ksteps, int bits, Visit visit) {
+  const size_t ck = (size_t)mgemv::chunk_k(bits);
+  const size_t tile = n / mgemv::kTileRows, r = n % mgemv::kTileRows;
+  size_t k0 = 0;
+  for (size_t s = 0; s < ksteps && k0 < k; ++s) {
+    const size_t unit = (tile * ksteps + s) * (size_t)mgemv::kUnitBytes;
+    for (size_t slice = 0; slice < (size_t)mgemv::kKSlices && k0 < k; ++slice) {
+      const size_t lane_off = (slice * mgemv::kTileRows + r) * (size_t)mgemv::kChunkBytes;
+      for (size_t blk = 0; blk < (size_t)mgemv::kBlocksPerUnit && k0 < k; ++blk, k0 += ck)
+        visit(k0 * (size_t)bits / 8, unit + blk * (size_t)mgemv::kBlockBytes + lane_off);
+    }
+  }
 }
 
 // One matrix: rows of k elements (n_out rows) -> tile layout.
 void tile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k, int bits) {
   const size_t ksteps = (size_t)mgemv::num_ksteps((int)k, bits);
-  const size_t ck = (size_t)mgemv::chunk_k(bits);
   const size_t row_bytes = k * (size_t)bits / 8;
-  std::memset(dst, 0, mgemv::preprocessed_bytes(n_out, k, bits));
+  // zero bytes only where the layout pads: whole rows past n_out, reduction positions past k
+  if (n_out % mgemv::kTileRows != 0 || k % (size_t)mgemv::step_k(bits) != 0) {
+    const size_t total = mgemv::preprocessed_bytes(n_out, k, bits), piece = (size_t)1 << 20;
+#pragma omp parallel for schedule(static)
+    for (long long off = 0; off < (long long)total; off += (long long)piece)
+      std::memset(dst + off, 0, total - (size_t)off < piece ? total - (size_t)off : piece);
+  }
 #pragma omp parallel for schedule(static)
   for (long long n = 0; n < (long long)n_out; ++n) {
     const uint8_t* row = src + (size_t)n * row_bytes;
-    for (size_t k0 = 0; k0 < k; k0 += ck) {
+    for_each_chunk_of_row((size_t)n, k, ksteps, bits, [&](size_t src_off, size_t dst_off) {
       uint32_t words[4];
-      std::memcpy(words, row + k0 * (size_t)bits / 8, mgemv::kChunkBytes);
-      for (int j = 0; j < 4; ++j)
-        words[j] = bits == 4 ? mgemv::encode_int4_word(words[j]) : mgemv::encode_int8_word(words[j]);
-      std::memcpy(dst + mgemv::chunk_offset((size_t)n, k0, ksteps, bits), words, mgemv::kChunkBytes);
-    }
+      std::memcpy(words, row + src_off, mgemv::kChunkBytes);
+      if (bits == 4) {
+        for (int j = 0; j < 4; ++j) words[j] = mgemv::encode_int4_word(words[j]);
+      } else {
+        for (int j = 0; j < 4; ++j) words[j] = mgemv::encode_int8_word(words[j]);
+      }
+      std::memcpy(dst + dst_off, words, mgemv::kChunkBytes);
+    });
   }
 }
 
 void untile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k, int bits) {
   const size_t ksteps = (size_t)mgemv::num_ksteps((int)k, bits);
-  const size_t ck = (size_t)mgemv::chunk_k(bits);
   const size_t row_bytes = k * (size_t)bits / 8;
 #pragma omp parallel for schedule(static)
   for (long long n = 0; n < (long long)n_out; ++n) {
     uint8_t* row = dst + (size_t)n * row_bytes;
-    for (size_t k0 = 0; k0 < k; k0 += ck) {
+    for_each_chunk_of_row((size_t)n, k, ksteps, bits, [&](size_t row_off, size_t tiled_off) {
       uint32_t words[4];
-      std::memcpy(words, src + mgemv::chunk_offset((size_t)n, k0, ksteps, bits), mgemv::kChunkBytes);
-      for (int j = 0; j < 4; ++j)
-        words[j] = bits == 4 ? mgemv::decode_int4_word(words[j]) : mgemv::decode_int8_word(words[j]);
-      std::memcpy(row + k0 * (size_t)bits / 8, words, mgemv::kChunkBytes);
-    }
+      std::memcpy(words, src + tiled_off, mgemv::kChunkBytes);
+      if (bits == 4) {
+        for (int j = 0; j < 4; ++j) words[j] = mgemv::decode_int4_word(words[j]);
+      } else {
+        for (int j = 0; j < 4; ++j) words[j] = mgemv::decode_int8_word(words[j]);
+      }
+      std::memcpy(row + row_off, words, mgemv::kChunkBytes);
+    });
   }
 }
 

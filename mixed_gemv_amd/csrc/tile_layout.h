@@ -95,15 +95,18 @@ MGEMV_HD uint32_t rotr32(uint32_t v, int s) { return s ? (v >> s) | (v << (32 - 
 MGEMV_HD int int4_field_shift(int e) {
   return e == 0 ? 7 : e == 1 ? 23 : e == 2 ? 3 : e == 3 ? 19 : e == 4 ? 15 : e == 5 ? 31 : e == 6 ? 11 : 27;
 }
+// Straight-line forms of "field e moves from bit 4e to bit int4_field_shift(e)" (the host
+// preprocessor spends its time here).
 MGEMV_HD uint32_t encode_int4_word(uint32_t natural) {
   const uint32_t b = natural ^ 0x88888888u;  // +8 on each two's-complement nibble
-  uint32_t w = 0;
-  for (int e = 0; e < 8; ++e) w |= rotl32((b >> (4 * e)) & 0xfu, int4_field_shift(e));
-  return w;
+  return ((b & 0x0000000fu) << 7) | ((b & 0x000000f0u) << 19) | ((b & 0x00000f00u) >> 5) | ((b & 0x0000f000u) << 7) |
+         ((b & 0x000f0000u) >> 1) | rotl32(b & 0x00f00000u, 11) | ((b & 0x0f000000u) >> 13) | ((b & 0xf0000000u) >> 1);
 }
 MGEMV_HD uint32_t decode_int4_word(uint32_t stored) {
-  uint32_t b = 0;
-  for (int e = 0; e < 8; ++e) b |= (rotr32(stored, int4_field_shift(e)) & 0xfu) << (4 * e);
+  const uint32_t w = stored;
+  const uint32_t b = ((w >> 7) & 0x0000000fu) | ((w >> 19) & 0x000000f0u) | ((w << 5) & 0x00000f00u) |
+                     ((w >> 7) & 0x0000f000u) | ((w << 1) & 0x000f0000u) | (rotr32(w, 11) & 0x00f00000u) |
+                     ((w << 13) & 0x0f000000u) | ((w << 1) & 0xf0000000u);
   return b ^ 0x88888888u;
 }
 MGEMV_HD uint32_t encode_int8_word(uint32_t natural) { return natural ^ 0x80808080u; }
