@@ -262,6 +262,9 @@ MGEMV_API int mgemv_tuned_plan_count(void);
  * out[6] = tiles per wave (matrix-core path), out[7] = most tiles a wave walks one after the
  * other (VALU path). */
 MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]);
+/* The same for the _bf16 entry points (their kernels are compiled for at most 8 waves per workgroup, and of
+ * the matrix-core kernels only the LDS-staged one exists for bf16). */
+MGEMV_API int mgemv_query_launch_bf16(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]);
 
 #ifdef __cplusplus
 }

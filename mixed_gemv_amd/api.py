@@ -257,11 +257,13 @@ def set_dequant_form(form=DEQUANT_AUTO):
     _lib.check(_lib.lib().mgemv_set_dequant_form(int(form)), "set_dequant_form")
 
 
-def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0):
-    """The geometry mgemv_gemv would use (group_size as passed to the GEMV; it only selects tuned plans)."""
+def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0, element="f16"):
+    """The geometry mgemv_gemv (element="bf16": mgemv_gemv_bf16) would use; group_size as passed to the GEMV
+    (it only selects tuned plans)."""
     out = (ctypes.c_int * 8)()
-    _lib.check(_lib.lib().mgemv_query_launch(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size),
-                                             ctypes.byref(out)), "query_launch")
+    fn = _lib.lib().mgemv_query_launch_bf16 if _is_bf16(element, None) else _lib.lib().mgemv_query_launch
+    _lib.check(fn(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size), ctypes.byref(out)),
+               "query_launch")
     keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave",
             "tiles_in_sequence")
     return dict(zip(keys, list(out)))

@@ -350,6 +350,19 @@ hipError_t launch_dequant(const DequantParams& p, int qop, half_t* out, hipStrea
   }
 }
 
+// The knobs of a problem with the element type taken into account.
+PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_batch, int act) {
+  PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch);
+  if (act == kActBf16) {
+    // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
+    // fp32 dequantiser wants the registers of 8-wave workgroups
+    if (num_tiles(n_out) < 2) knobs.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1;
+    knobs.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
+    knobs.wide_waves = true;
+  }
+  return knobs;
+}
+
 // act: kActF16 or kActBf16, the type behind every 16-bit operand.
 int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
              const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k, int group_size,
@@ -371,15 +384,7 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
   g.n_out = n_out;
   g.k = k;
   g.group_size = group_size;
-  PlanKnobs knobs = knobs_for(n_out, k, weight_bits, group_size, m_batch);
-  if (act == kActBf16) {
-    // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
-    // fp32 dequantiser wants the registers of 8-wave workgroups
-    if (num_tiles(n_out) < 2) knobs.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1;
-    knobs.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
-    knobs.wide_waves = true;
-  }
-  g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs);
+  g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act));
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
@@ -579,12 +584,25 @@ int mgemv_tuned_plan_clear(void) {
 
 int mgemv_tuned_plan_count(void) { return mgemv::g_tuned_count.load(); }
 
+namespace {
+int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_size, int act, int out[8]);
+}
+
 int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]) {
+  return query_launch_any(n_out, m_batch, k, weight_bits, group_size, mgemv::kActF16, out);
+}
+
+int mgemv_query_launch_bf16(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]) {
+  return query_launch_any(n_out, m_batch, k, weight_bits, group_size, mgemv::kActBf16, out);
+}
+
+namespace {
+int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_size, int act, int out[8]) {
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   const int st = check_tuned_key(n_out, k, weight_bits, group_size, m_batch);
   if (st != MGEMV_OK) return st;
-  const mgemv::LaunchPlan lp = mgemv::plan_launch(n_out, k, weight_bits, m_batch,
-                                                  mgemv::knobs_for(n_out, k, weight_bits, group_size, m_batch));
+  const mgemv::LaunchPlan lp = mgemv::plan_launch(
+      n_out, k, weight_bits, m_batch, mgemv::knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act));
   out[0] = lp.wgs_per_xcd * mgemv::kNumXcd;
   out[1] = lp.threads;
   out[2] = lp.split_k;
@@ -595,5 +613,6 @@ int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group
   out[7] = lp.tiles_in_sequence;
   return MGEMV_OK;
 }
+}  // namespace
 
 }  // extern "C"

@@ -162,6 +162,15 @@ def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
             assert ulp <= MAX_ULP and differing <= MAX_DIFFERING, (m_batch, ulp, differing)
 
 
+def test_launch_query_knows_the_bf16_kernels(gpu):
+    # 8-wave workgroups at most, and only the LDS-staged matrix-core kernel
+    assert mg.query_launch(1024, 1, 8192, 4, 128)["threads"] == 1024
+    assert mg.query_launch(1024, 1, 8192, 4, 128, element="bf16")["threads"] == 512
+    assert mg.query_launch(1024, 5, 2048, 4, 128)["matrix_core"] == 1
+    assert mg.query_launch(1024, 5, 2048, 4, 128, element="bf16")["matrix_core"] == 2
+    assert mg.query_launch(16, 7, 512, 4, 128, element="bf16")["matrix_core"] == 0      # a single tile
+
+
 def test_batched_launch_with_strides(gpu):
     """batch_count problems in one launch: stacked weights and scales, shared activations."""
     import torch
