@@ -146,8 +146,8 @@ def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
             for form in (mg.DEQUANT_AUTO, mg.DEQUANT_EXACT_INTEGER):
                 mg.set_dequant_form(form)
                 mg.set_matrix_core_threshold(1)
-                for split in (0, 1, 2):
-                    mg.set_launch_override(split, 0, 0, 0)
+                for split, tw in ((0, 0), (1, 2), (2, 2), (4, 1), (2, 4), (1, 8)):   # k-split waves, tiles per workgroup
+                    mg.set_launch_override(split, tw, 0, 0)
                     results.append(dev.run().copy())
                     assert np.array_equal(results[-1], dev.run())   # reproducible
                 mg.set_launch_override(0, 0, 0, 0)

@@ -360,11 +360,18 @@ def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
         results = []
         try:
             mg.set_matrix_core_threshold(1)
-            for variant, split in ((mg.MATRIX_CORE_LDS_STAGED, 0), (mg.MATRIX_CORE_LDS_STAGED, 1),
-                                   (mg.MATRIX_CORE_LDS_STAGED, 2), (mg.MATRIX_CORE_REGISTER_OPERAND, 0)):
+            # (variant, k-split waves, tiles per workgroup): 1-8 tiles share an activation stage of 8 or 16
+            # rows; 7 tiles do not divide by 2, 4 or 8, so some waves of the last workgroup have no tile
+            for variant, split, tw in ((mg.MATRIX_CORE_LDS_STAGED, 0, 0), (mg.MATRIX_CORE_LDS_STAGED, 1, 2),
+                                       (mg.MATRIX_CORE_LDS_STAGED, 2, 2), (mg.MATRIX_CORE_LDS_STAGED, 4, 1),
+                                       (mg.MATRIX_CORE_LDS_STAGED, 2, 4), (mg.MATRIX_CORE_LDS_STAGED, 1, 8),
+                                       (mg.MATRIX_CORE_REGISTER_OPERAND, 0, 0)):
                 mg.set_matrix_core_variant(variant)
-                mg.set_launch_override(split, 0, 0, 0)
-                assert mg.query_launch(n_out, m_batch, k, bits)["matrix_core"] == (2 if variant == mg.MATRIX_CORE_LDS_STAGED else 1)
+                mg.set_launch_override(split, tw, 0, 0)
+                plan = mg.query_launch(n_out, m_batch, k, bits)
+                assert plan["matrix_core"] == (2 if variant == mg.MATRIX_CORE_LDS_STAGED else 1)
+                if variant == mg.MATRIX_CORE_LDS_STAGED and tw and (8 if m_batch <= 8 else 16) // tw >= 2:
+                    assert plan["tiles_per_wg"] == tw, plan
                 results.append(dev.run().copy())
                 assert np.array_equal(results[-1].view(np.uint16), dev.run().view(np.uint16))   # reproducible
             mg.set_matrix_core_threshold(17)
