@@ -184,21 +184,31 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     LaunchPlan lp{};
     lp.matrix_core = true;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
-    // Tiles per workgroup = waves that share one activation stage: as many as still leave about
-    // 170 workgroups (two thirds of the compute units), at most 8 and at most half the staged rows.
+    // Tiles per workgroup = waves that share one activation stage: as few as bring the launch down
+    // to one workgroup per compute unit or fewer, at most 8 and at most half the staged rows.
     // Measured, 16 rows: 4096x4096 (256 tiles) 6.3 us at 1 tile against 7.2 at 2; 8192x8192 (512)
     // 13.4 at 2 against 17.8 at 4; 11008x4096 (688) 10.1 at 4 against 11.3 at 2 and 14.2 at 8;
     // 28672x8192 (1792) 28.3 at 8 against 30.6 at 4 and 32.8 at 2.  8 rows: 4096x4096 5.4 at 1
-    // against 6.4 at 2; 11008x4096 9.0 at 4 against 9.7 at 2; 28672x8192 27.6 at 4 against 29.5 at 2.
+    // against 6.4 at 2; 5120x5120 (320) 7.7 at 2 against 9.3 at 1; 10240x8192 (640) 14.7 at 4
+    // against 15.5 at 2; 11008x4096 9.0 at 4 against 9.7 at 2; 28672x8192 27.6 at 4 against 29.5 at 2.
     lp.tiles_per_wg = 1;
-    for (int tw = 2; tw <= 8 && tw * 2 <= lp.staged_rows; tw *= 2)
-      if (ceil_div(tiles, tw) >= 170) lp.tiles_per_wg = tw;
+    while (ceil_div(tiles, lp.tiles_per_wg) > kNumCus && lp.tiles_per_wg * 2 <= 8 &&
+           lp.tiles_per_wg * 4 <= lp.staged_rows)
+      lp.tiles_per_wg *= 2;
     // the kernel exists for 2, 4, 8 or 16 staged rows per wave of a k range
     if (ov_tw > 0 && ov_tw <= 8 && lp.staged_rows % ov_tw == 0 && lp.staged_rows / ov_tw >= 2) lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
     const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;
     while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 2048) split *= 2;
+    // A split that leaves the last wave nearly idle (10 k steps over 4 waves: 3, 3, 3, 1) loses
+    // to half as many evenly loaded waves, as long as the workgroup keeps four (5120x5120, 8 rows,
+    // 2 tiles: 7.6 us at 2 waves per tile against 8.1 at 4; 6912x5120, 16 rows: 9.0 against 9.6;
+    // but 4096x6656, 8 rows, 1 tile: 9.1 at 2 against 7.8 at 4).
+    auto padded_steps = [&](int s) { const int st = ceil_div(ksteps, s); return st * ceil_div(ksteps, st); };
+    if (lp.tiles_per_wg * split >= 8 && padded_steps(split) * 100 > ksteps * 115 &&
+        padded_steps(split / 2) < padded_steps(split))
+      split /= 2;
     if (ov_sk > 0) split = ov_sk > max_split ? max_split : ov_sk;
     if (split > ksteps) split = ksteps;
     lp.steps_per_wave = ceil_div(ksteps, split);
@@ -238,7 +248,16 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     if (mc) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
   } else {
     constexpr int kWaveBudget = 8192;
+    constexpr int kSimds = kNumCus * 4;
     split_k = ksteps < max_waves ? ksteps : max_waves;
+    // One wave per unit does not fit the machine at once, and one wave per tile fills at least
+    // 80 % of the SIMDs of its last round: the whole-k waves win (13824x5120: 9.1 us against
+    // 10.3 at 5 waves per tile; 27648x5120: 15.6 against 17.5 at 3; 14848x6144: 10.6 against 12.1
+    // at 6; 13824x8192: 12.6 against 13.7 at 8).  With a worse fit they lose (17408x5120, 1088
+    // tiles: 13.8 against 12.4), and the halving below stands.
+    const bool whole_k_waves = !mc && (long long)groups * split_k > kWaveBudget &&
+                               (long long)tiles * 100 >= (long long)ceil_div(tiles, kSimds) * kSimds * 80;
+    if (whole_k_waves) split_k = 1;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
     if (!mc && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
         (long long)groups * ((split_k + 1) / 2) >= 4096)
