@@ -195,6 +195,19 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     while (ceil_div(tiles, lp.tiles_per_wg) > kNumCus && lp.tiles_per_wg * 2 <= 8 &&
            lp.tiles_per_wg * 4 <= lp.staged_rows)
       lp.tiles_per_wg *= 2;
+    // Still more workgroups than compute units: a count just above a multiple of 256 leaves most
+    // of the last round idle, and halving the tiles per workgroup evens that out (18944x3584,
+    // 8 rows: 296 workgroups of 4 tiles 12.8 us, 592 of 2 tiles 11.8; 22016x4096: 14.4 / 13.3).
+    // Largest count whose last round is at least three quarters full.
+    if (ceil_div(tiles, lp.tiles_per_wg) > kNumCus) {
+      for (int tw = lp.tiles_per_wg; tw >= 1; tw /= 2) {
+        const int wgs = ceil_div(tiles, tw);
+        if (wgs * 4 >= ceil_div(wgs, kNumCus) * kNumCus * 3) {
+          lp.tiles_per_wg = tw;
+          break;
+        }
+      }
+    }
     // the kernel exists for 2, 4, 8 or 16 staged rows per wave of a k range
     if (ov_tw > 0 && ov_tw <= 8 && lp.staged_rows % ov_tw == 0 && lp.staged_rows / ov_tw >= 2) lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
@@ -245,9 +258,18 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // 16 k steps (1024x4096: 3.38 us against 3.54; 1024x8192: 4.54 against 4.77); with a longer
     // reduction it is not (2048x11008: 6.35 at 8 waves against 6.12).
     if (!mc && tiles <= 128 && ksteps <= 16) split_k = ksteps;
+    // More than one workgroup per compute unit and 5-8 k steps, one row: four waves would take
+    // two units each, the one length at which the two-deep pipeline overlaps nothing; one unit
+    // per wave is 6-7 % ahead (4608x4096: 4.81 us against 5.13; 6144x4096: 4.98 against 5.29),
+    // while at 256 tiles four waves win (4096x4096: 4.08 against 4.33).
+    if (!mc && m_batch == 1 && tiles > kNumCus && ceil_div(ksteps, 4) == 2) split_k = ksteps;
     if (mc) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
   } else {
-    constexpr int kWaveBudget = 8192;
+    // One row and up to 8 k steps: workgroups of up to 8 one-unit waves stay ahead of two-unit
+    // waves well past 8192 waves (22016x4096, 11008 waves: 10.9 us against 11.8; 27200x4096,
+    // 13600 waves: 12.6 against 13.0; 36864x2560: 11.8 against 12.3).
+    const bool short_single_row = !mc && m_batch == 1 && ksteps <= 8;
+    const int kWaveBudget = short_single_row ? 16384 : 8192;
     constexpr int kSimds = kNumCus * 4;
     split_k = ksteps < max_waves ? ksteps : max_waves;
     // One wave per unit does not fit the machine at once, and one wave per tile fills at least
@@ -259,7 +281,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
                                (long long)tiles * 100 >= (long long)ceil_div(tiles, kSimds) * kSimds * 80;
     if (whole_k_waves) split_k = 1;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
-    if (!mc && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
+    if (!mc && !short_single_row && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
         (long long)groups * ((split_k + 1) / 2) >= 4096)
       split_k = (split_k + 1) / 2;
   }
