@@ -174,8 +174,8 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
                                         int max_workgroups);
 
 /* Smallest m_batch served by the matrix-core kernels instead of the VALU kernel.  0 restores the
- * built-in rule (from 5 rows; from 4 rows on matrices of 8192 or more 16-row x 512-k units; from
- * 3 rows on 16384 or more units; from 2 rows on 24576 or more units; never for a single row); 17 keeps every batch size on the VALU kernel.  For tuning and tests.  Process-wide. */
+ * built-in rule (from 5 rows; from 3 rows on matrices of more than 256 16-row tiles, n_out > 4096;
+ * from 2 rows on 1536 or more tiles; never for a single row); 17 keeps every batch size on the VALU kernel.  For tuning and tests.  Process-wide. */
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Which of the two matrix-core kernels serves the small batches:

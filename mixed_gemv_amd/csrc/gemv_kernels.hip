@@ -155,10 +155,16 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 //   8192x8192 (8 k units):   3 rows 10.8 / 11.2, 4 rows 11.8 / 11.2
 //   28672x8192 (28 k units): 2 rows 27.5 / 26.2, 3 rows 31.9 / 26.7
 // From 5 rows the VALU kernel would need a second launch.
-inline bool use_matrix_cores(int m_batch, long long units, int forced) {
+// Which row counts go to the matrix cores.  The VALU kernel pays per row, the matrix-core kernels
+// (almost) not, but the VALU kernel is at its best with at most one workgroup per compute unit:
+// measured over 21 shapes, 3 and 4 rows are faster on the matrix cores whenever there are more
+// than 256 tiles (5120x4096, 3 rows: 6.45 us against 6.74; 14336x4096, 4 rows: 9.2 against 11.4;
+// the one exception found, 11008x4096 at 3 rows, loses 5 %) and on the VALU kernel below that
+// (4096x14336, 4 rows: 10.6 against 11.3); 2 rows only from about 1536 tiles (32000x4096: 15.1
+// against 16.4; 28672x8192: 25.9 against 27.3; 10240x8192: 14.2 against 12.7 the other way).
+inline bool use_matrix_cores(int m_batch, int tiles, long long units, int forced) {
   if (forced > 0) return m_batch >= forced;
-  return m_batch >= 5 || (m_batch >= 4 && units >= 8192) || (m_batch >= 3 && units >= 16384) ||
-         (m_batch >= 2 && units >= 24576);
+  return m_batch >= 5 || (m_batch >= 3 && tiles > kNumCus && units >= 2048) || (m_batch >= 2 && tiles >= 1536);
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -167,7 +173,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
-  const bool mc = use_matrix_cores(m_batch, (long long)tiles * ksteps, knobs.matrix_core_min_batch);
+  const bool mc = use_matrix_cores(m_batch, tiles, (long long)tiles * ksteps, knobs.matrix_core_min_batch);
   // Small problems (up to 256 tiles) with few rows or a short reduction take the register-operand
   // kernel with one tile per wave: a lane of a row past m_batch loads nothing there, and no barrier
   // ties the waves of a workgroup together (1024x2048, 5 rows: 3.4 us against 4.6 us LDS-staged;
@@ -277,7 +283,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // 10.3 at 5 waves per tile; 27648x5120: 15.6 against 17.5 at 3; 14848x6144: 10.6 against 12.1
     // at 6; 13824x8192: 12.6 against 13.7 at 8).  With a worse fit they lose (17408x5120, 1088
     // tiles: 13.8 against 12.4), and the halving below stands.
-    const bool whole_k_waves = !mc && (long long)groups * split_k > kWaveBudget &&
+    const bool whole_k_waves = !mc && m_batch <= 2 && (long long)groups * split_k > kWaveBudget &&
                                (long long)tiles * 100 >= (long long)ceil_div(tiles, kSimds) * kSimds * 80;
     if (whole_k_waves) split_k = 1;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
