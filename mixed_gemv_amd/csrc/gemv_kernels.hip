@@ -264,17 +264,17 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // 16 k steps (1024x4096: 3.38 us against 3.54; 1024x8192: 4.54 against 4.77); with a longer
     // reduction it is not (2048x11008: 6.35 at 8 waves against 6.12).
     if (!mc && tiles <= 128 && ksteps <= 16) split_k = ksteps;
-    // More than one workgroup per compute unit and 5-8 k steps, one row: four waves would take
+    // More than one workgroup per compute unit and 5-8 k steps, one or two rows: four waves would take
     // two units each, the one length at which the two-deep pipeline overlaps nothing; one unit
     // per wave is 6-7 % ahead (4608x4096: 4.81 us against 5.13; 6144x4096: 4.98 against 5.29),
     // while at 256 tiles four waves win (4096x4096: 4.08 against 4.33).
-    if (!mc && m_batch == 1 && tiles > kNumCus && ceil_div(ksteps, 4) == 2) split_k = ksteps;
+    if (!mc && m_batch <= 2 && tiles > kNumCus && ceil_div(ksteps, 4) == 2) split_k = ksteps;
     if (mc) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
   } else {
-    // One row and up to 8 k steps: workgroups of up to 8 one-unit waves stay ahead of two-unit
+    // One or two rows and up to 8 k steps: workgroups of up to 8 one-unit waves stay ahead of two-unit
     // waves well past 8192 waves (22016x4096, 11008 waves: 10.9 us against 11.8; 27200x4096,
     // 13600 waves: 12.6 against 13.0; 36864x2560: 11.8 against 12.3).
-    const bool short_single_row = !mc && m_batch == 1 && ksteps <= 8;
+    const bool short_single_row = !mc && m_batch <= 2 && ksteps <= 8;
     const int kWaveBudget = short_single_row ? 16384 : 8192;
     constexpr int kSimds = kNumCus * 4;
     split_k = ksteps < max_waves ? ksteps : max_waves;
