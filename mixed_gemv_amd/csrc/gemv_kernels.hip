@@ -161,10 +161,14 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 // than 256 tiles (5120x4096, 3 rows: 6.45 us against 6.74; 14336x4096, 4 rows: 9.2 against 11.4;
 // the one exception found, 11008x4096 at 3 rows, loses 5 %) and on the VALU kernel below that
 // (4096x14336, 4 rows: 10.6 against 11.3); 2 rows only from about 1536 tiles (32000x4096: 15.1
-// against 16.4; 28672x8192: 25.9 against 27.3; 10240x8192: 14.2 against 12.7 the other way).
-inline bool use_matrix_cores(int m_batch, int tiles, long long units, int forced) {
+// against 16.4; 28672x8192: 25.9 against 27.3; 10240x8192: 14.2 against 12.7 the other way), and
+// with fewer than 8 k steps only when one-unit VALU waves would not fit the machine (50304x2048,
+// 12576 units: 15.2 against 12.8 the other way; 151936x2048, 37984 units: 33.1 against 35.1).
+inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced) {
   if (forced > 0) return m_batch >= forced;
-  return m_batch >= 5 || (m_batch >= 3 && tiles > kNumCus && units >= 2048) || (m_batch >= 2 && tiles >= 1536);
+  const long long units = (long long)tiles * ksteps;
+  return m_batch >= 5 || (m_batch >= 3 && tiles > kNumCus && units >= 2048) ||
+         (m_batch >= 2 && tiles >= 1536 && (ksteps >= 8 || units > 16384));
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -173,7 +177,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
-  const bool mc = use_matrix_cores(m_batch, tiles, (long long)tiles * ksteps, knobs.matrix_core_min_batch);
+  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch);
   // Small problems (up to 256 tiles) with few rows or a short reduction take the register-operand
   // kernel with one tile per wave: a lane of a row past m_batch loads nothing there, and no barrier
   // ties the waves of a workgroup together (1024x2048, 5 rows: 3.4 us against 4.6 us LDS-staged;
