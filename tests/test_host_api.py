@@ -304,3 +304,61 @@ def test_adaptor_mirror_rejects_small_groups_like_the_reference():
     with pytest.raises(MixedGemvError) as ei:
         mg.GemvAdaptor().initialize(args)
     assert ei.value.status == 5
+
+
+# (n_out, m_batch, k) -> expected fields of the built-in plan, int4 group 128.  Each row is a shape
+# on which the rule that produces it was measured against its alternatives on an MI355X; the
+# test pins the rules, so a change to plan_launch that moves one of them shows up here.
+BUILTIN_PLANS = [
+    # exact fit: one 4-wave workgroup per compute unit, every wave walking 7 tiles
+    ((28672, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256, split_k=4, tiles_in_sequence=7)),
+    ((8192, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256)),
+    # at most one workgroup per compute unit: four k-split waves
+    ((4096, 1, 4096), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=2)),
+    ((4096, 1, 14336), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=7)),
+    # few tiles and a short reduction: one unit per wave
+    ((1024, 1, 4096), dict(matrix_core=0, split_k=8, steps_per_wave=1)),
+    # more than one workgroup per compute unit and 5-8 k steps: one unit per wave, at one and two rows
+    ((6144, 1, 4096), dict(matrix_core=0, workgroups=384, split_k=8, steps_per_wave=1)),
+    ((6144, 2, 4096), dict(matrix_core=0, workgroups=384, split_k=8, steps_per_wave=1)),
+    ((22016, 1, 4096), dict(matrix_core=0, workgroups=1376, split_k=8, steps_per_wave=1)),
+    # one wave per unit would not fit and one wave per tile fills the SIMDs: whole-k waves
+    ((13824, 1, 5120), dict(matrix_core=0, workgroups=864, threads=64, split_k=1, steps_per_wave=10)),
+    ((128256, 1, 4096), dict(matrix_core=0, workgroups=8016, threads=64, split_k=1)),
+    # ... and with a poor fit the k split stays
+    ((17408, 1, 5120), dict(matrix_core=0, workgroups=1088, split_k=5, steps_per_wave=2)),
+    # matrix cores: from 5 rows anywhere, from 3 rows on more than 256 tiles, from 2 rows on many tiles
+    ((4096, 4, 4096), dict(matrix_core=0)),
+    ((4096, 5, 4096), dict(matrix_core=1)),
+    ((4096, 8, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
+    ((5120, 3, 4096), dict(matrix_core=2)),
+    ((4096, 4, 14336), dict(matrix_core=0)),
+    ((10240, 2, 8192), dict(matrix_core=0)),
+    ((28672, 2, 8192), dict(matrix_core=2)),
+    ((50304, 2, 2048), dict(matrix_core=0)),
+    ((151936, 2, 2048), dict(matrix_core=2)),
+    # tiles that share an activation stage: as few as give at most 256 workgroups ...
+    ((5120, 8, 5120), dict(matrix_core=2, tiles_per_wg=2, workgroups=160, split_k=2, steps_per_wave=5)),
+    ((8192, 16, 8192), dict(matrix_core=2, tiles_per_wg=2, workgroups=256, split_k=4)),
+    ((10240, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=160)),
+    ((28672, 16, 8192), dict(matrix_core=2, tiles_per_wg=8, workgroups=224, split_k=1)),
+    # ... or, when that cannot be had, a count whose last round of 256 is well filled
+    ((28672, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=448)),
+    ((18944, 8, 3584), dict(matrix_core=2, tiles_per_wg=2, workgroups=592, split_k=1)),
+    # an uneven k split is halved only while the workgroup keeps four waves
+    ((4096, 8, 6656), dict(matrix_core=2, tiles_per_wg=1, split_k=4, steps_per_wave=4)),
+    ((8192, 8, 6656), dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=7)),
+]
+
+
+@pytest.mark.parametrize("shape,want", BUILTIN_PLANS, ids=[f"{s[0]}x{s[2]}_m{s[1]}" for s, _ in BUILTIN_PLANS])
+def test_builtin_launch_rules_on_the_shapes_they_were_measured_on(shape, want):
+    n_out, m_batch, k = shape
+    got = mg.query_launch(n_out, m_batch, k, 4, 128)
+    assert {key: got[key] for key in want} == want, got
+    # every plan covers every tile and every k step, within the workgroup size the kernels allow
+    tiles, ksteps = -(-n_out // 16), -(-k // 512)
+    assert got["split_k"] * got["steps_per_wave"] >= ksteps > (got["split_k"] - 1) * got["steps_per_wave"]
+    assert got["threads"] <= 1024 and got["threads"] % 64 == 0
+    per_workgroup = got["tiles_per_wg"] * got["tiles_per_wave"] * got["tiles_in_sequence"]
+    assert got["workgroups"] * per_workgroup >= tiles
