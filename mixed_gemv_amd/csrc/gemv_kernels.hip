@@ -150,12 +150,8 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
   return it == g_tuned_plans.end() ? kn : it->second;
 }
 
-// Built-in rule, measured (VALU kernel against the matrix-core kernel the plan would pick, us):
-//   4096x4096 (2 k units):   4 rows 5.2 / 5.5,   5 rows 8.8 / 5.5
-//   8192x8192 (8 k units):   3 rows 10.8 / 11.2, 4 rows 11.8 / 11.2
-//   28672x8192 (28 k units): 2 rows 27.5 / 26.2, 3 rows 31.9 / 26.7
-// From 5 rows the VALU kernel would need a second launch.
-// Which row counts go to the matrix cores.  The VALU kernel pays per row, the matrix-core kernels
+// Which row counts go to the matrix cores.  From 5 rows the VALU kernel would need a second pass
+// over the weights (4096x4096: 8.8 us against 5.5).  The VALU kernel pays per row, the matrix-core kernels
 // (almost) not, but the VALU kernel is at its best with at most one workgroup per compute unit:
 // measured over 21 shapes, 3 and 4 rows are faster on the matrix cores whenever there are more
 // than 256 tiles (5120x4096, 3 rows: 6.45 us against 6.74; 14336x4096, 4 rows: 9.2 against 11.4;
