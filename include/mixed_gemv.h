@@ -237,7 +237,8 @@ MGEMV_API int mgemv_fold_zero_points_bf16(uint16_t *out, const uint16_t *scales,
  * (0 = built-in rule for that knob); `kernel` picks the kernel.  A process-wide override that is
  * set (mgemv_set_launch_override, _matrix_core_threshold, _matrix_core_variant) takes precedence
  * over the table.  Setting an existing key replaces it.  Results never depend on the plan beyond
- * the order of the fp32 partial sums.  Thread-safe. */
+ * the order of the fp32 partial sums.  The fp16 and the _bf16 entry points share the table (a bf16
+ * launch clamps an entry to what its kernels allow).  Thread-safe. */
 enum {
   MGEMV_KERNEL_AUTO = 0,
   MGEMV_KERNEL_VALU = 1,
