@@ -480,6 +480,31 @@ def test_vocabulary_projection_one_tile_per_workgroup(gpu):
     check(prob, gpu, dequant=False)
 
 
+# Shapes on which the remaining launch rules were measured, each with the plan field that shows the
+# rule took effect: whole-k single-wave workgroups, one-unit waves at 5-8 k steps (in and over the
+# usual wave count), matrix cores from 3 rows, the tile count per activation stage and the balanced
+# k split of the LDS-staged kernel.
+RULES = [
+    ("whole_k_m1", 13824, 5120, 1, dict(matrix_core=0, threads=64, split_k=1, steps_per_wave=10)),
+    ("whole_k_m2", 13824, 5120, 2, dict(matrix_core=0, threads=64, split_k=1)),
+    ("one_unit_waves_m2", 6144, 4096, 2, dict(matrix_core=0, split_k=8, steps_per_wave=1)),
+    ("one_unit_waves_11008_waves", 22016, 4096, 1, dict(matrix_core=0, split_k=8, workgroups=1376)),
+    ("matrix_cores_at_3_rows", 5120, 4096, 3, dict(matrix_core=2)),
+    ("two_tiles_even_split", 5120, 5120, 8, dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=5)),
+    ("two_tiles_592_workgroups", 18944, 3584, 8, dict(matrix_core=2, tiles_per_wg=2, workgroups=592)),
+    ("four_tiles_160_workgroups", 10240, 8192, 8, dict(matrix_core=2, tiles_per_wg=4, workgroups=160)),
+]
+
+
+@pytest.mark.parametrize("cfg", RULES, ids=[c[0] for c in RULES])
+def test_launch_rule_shapes_full_size(gpu, cfg):
+    tag, n_out, k, mb, want = cfg
+    plan = mg.query_launch(n_out, mb, k, 4, 128)
+    assert {key: plan[key] for key in want} == want, plan
+    prob = Problem(tag, n_out, k, 4, SCALE_AND_ZEROS, 128, m_batch=mb, bias=(mb % 2 == 0), x_dist="normal")
+    check(prob, gpu, dequant=False)
+
+
 @pytest.mark.parametrize("cfg", FULL, ids=[c[0] for c in FULL])
 def test_baseline_configs_full_size(gpu, cfg):
     tag, n_out, k, bits, qop, g, mb, bias, xd, sr = cfg
