@@ -322,6 +322,11 @@ BUILTIN_PLANS = [
     ((6144, 1, 4096), dict(matrix_core=0, workgroups=384, split_k=8, steps_per_wave=1)),
     ((6144, 2, 4096), dict(matrix_core=0, workgroups=384, split_k=8, steps_per_wave=1)),
     ((22016, 1, 4096), dict(matrix_core=0, workgroups=1376, split_k=8, steps_per_wave=1)),
+    # 288-384 tiles and 9 or more k steps: two tiles per workgroup with two (from 20 k steps: four) waves each
+    ((5120, 1, 5120), dict(matrix_core=0, workgroups=160, tiles_per_wg=2, split_k=2, steps_per_wave=5)),
+    ((6144, 2, 8192), dict(matrix_core=0, workgroups=192, tiles_per_wg=2, split_k=2, steps_per_wave=8)),
+    ((5120, 1, 14336), dict(matrix_core=0, workgroups=160, tiles_per_wg=2, split_k=4, steps_per_wave=7)),
+    ((4160, 1, 8192), dict(matrix_core=0, tiles_per_wg=1, split_k=4)),
     # one wave per unit would not fit and one wave per tile fills the SIMDs: whole-k waves
     ((13824, 1, 5120), dict(matrix_core=0, workgroups=864, threads=64, split_k=1, steps_per_wave=10)),
     ((128256, 1, 4096), dict(matrix_core=0, workgroups=8016, threads=64, split_k=1)),
