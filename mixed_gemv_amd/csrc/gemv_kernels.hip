@@ -258,8 +258,16 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
                         : m_batch >= 3 || knobs.wide_waves ? kMaxWavesPerWideWorkgroup
                                                   : kMaxWavesPerWorkgroup;
   int split_k;
-  bool pair_tiles = false;
-  if (groups <= 384) {
+  // 288-512 tiles and a longer reduction: two tiles per workgroup, two k-split waves each (four
+  // up to 384 tiles from 20 k steps) -- at most one workgroup per compute unit and one wave per
+  // SIMD, the exact fit below without its divisibility -- beat one tile per workgroup with four
+  // waves (5120x5120: 5.8 us against 6.2; 6144x8192: 7.7 against 8.3; 5120x14336: 11.0 against
+  // 11.5) and one-unit or two-unit waves (7168x8192: 7.8 against 8.7; 6656x11008: 9.9 against
+  // 11.3; 7168x14336: 11.8 against 15.3); at 260 tiles they are 1-3 % behind (4160x8192).
+  const bool pair_tiles = !mc && tiles * 8 >= kNumCus * 9 && tiles <= 2 * kNumCus && ksteps >= 9;
+  if (pair_tiles) {
+    split_k = tiles <= 384 && ksteps >= 20 ? 4 : 2;
+  } else if (groups <= 384) {
     split_k = ksteps < 4 ? ksteps : 4;
     // With workgroups for at most half the compute units, one unit per wave is 4-5 % ahead up to
     // 16 k steps (1024x4096: 3.38 us against 3.54; 1024x8192: 4.54 against 4.77); with a longer
@@ -270,15 +278,6 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // per wave is 6-7 % ahead (4608x4096: 4.81 us against 5.13; 6144x4096: 4.98 against 5.29),
     // while at 256 tiles four waves win (4096x4096: 4.08 against 4.33).
     if (!mc && m_batch <= 2 && tiles > kNumCus && ceil_div(ksteps, 4) == 2) split_k = ksteps;
-    // 288-384 tiles and a longer reduction: two tiles per workgroup, two k-split waves each (four
-    // from 20 k steps) -- again at most one workgroup per compute unit and one wave per SIMD -- are
-    // 3-7 % ahead of one tile with four waves (5120x5120: 5.8 us against 6.2; 5120x8192: 7.6
-    // against 8.0; 6144x8192: 7.7 against 8.3; 5120x14336: 11.0 against 11.5); at 260 tiles they
-    // are 1-3 % behind (4160x8192).
-    if (!mc && tiles * 8 >= kNumCus * 9 && ksteps >= 9) {
-      split_k = ksteps >= 20 ? 4 : 2;
-      pair_tiles = true;
-    }
     if (mc) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
   } else {
     // One or two rows and up to 8 k steps: workgroups of up to 8 one-unit waves stay ahead of two-unit

@@ -322,7 +322,9 @@ BUILTIN_PLANS = [
     ((6144, 1, 4096), dict(matrix_core=0, workgroups=384, split_k=8, steps_per_wave=1)),
     ((6144, 2, 4096), dict(matrix_core=0, workgroups=384, split_k=8, steps_per_wave=1)),
     ((22016, 1, 4096), dict(matrix_core=0, workgroups=1376, split_k=8, steps_per_wave=1)),
-    # 288-384 tiles and 9 or more k steps: two tiles per workgroup with two (from 20 k steps: four) waves each
+    # 288-512 tiles and 9 or more k steps: two tiles per workgroup with two waves each (four up to 384 tiles from 20 k steps)
+    ((7168, 1, 14336), dict(matrix_core=0, workgroups=224, tiles_per_wg=2, split_k=2, steps_per_wave=14)),
+    ((7680, 1, 4096), dict(matrix_core=0, workgroups=480, tiles_per_wg=1, split_k=8)),
     ((5120, 1, 5120), dict(matrix_core=0, workgroups=160, tiles_per_wg=2, split_k=2, steps_per_wave=5)),
     ((6144, 2, 8192), dict(matrix_core=0, workgroups=192, tiles_per_wg=2, split_k=2, steps_per_wave=8)),
     ((5120, 1, 14336), dict(matrix_core=0, workgroups=160, tiles_per_wg=2, split_k=4, steps_per_wave=7)),
