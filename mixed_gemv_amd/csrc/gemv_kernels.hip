@@ -299,6 +299,10 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     if (!mc && !short_single_row && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
         (long long)groups * ((split_k + 1) / 2) >= 4096)
       split_k = (split_k + 1) / 2;
+    // From 16 k steps four waves with longer pipelines are level with or ahead of more, shorter
+    // ones (9216x14336: 16.9 us against 18.1 at 7 waves; 10240x11008: 14.8 against 15.3 at 11;
+    // 10240x8192 and 11008x8192: level).
+    if (!mc && ksteps >= 16 && split_k > 4) split_k = 4;
   }
   int tiles_per_wg = pair_tiles ? 2 : 1;
   int workgroup_cap = 0;

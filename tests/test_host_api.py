@@ -329,6 +329,8 @@ BUILTIN_PLANS = [
     ((6144, 2, 8192), dict(matrix_core=0, workgroups=192, tiles_per_wg=2, split_k=2, steps_per_wave=8)),
     ((5120, 1, 14336), dict(matrix_core=0, workgroups=160, tiles_per_wg=2, split_k=4, steps_per_wave=7)),
     ((4160, 1, 8192), dict(matrix_core=0, tiles_per_wg=1, split_k=4)),
+    # above 512 tiles and from 16 k steps: at most four k-split waves
+    ((9216, 1, 14336), dict(matrix_core=0, workgroups=576, tiles_per_wg=1, split_k=4, steps_per_wave=7)),
     # one wave per unit would not fit and one wave per tile fills the SIMDs: whole-k waves
     ((13824, 1, 5120), dict(matrix_core=0, workgroups=864, threads=64, split_k=1, steps_per_wave=10)),
     ((128256, 1, 4096), dict(matrix_core=0, workgroups=8016, threads=64, split_k=1)),
