@@ -382,9 +382,22 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
     const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
     const ConvertRegs c = make_convert_regs();
+    // With two or more activation rows, a wave of exactly two units runs straight-line code: the
+    // second unit is requested without waiting for the first and nothing is prefetched past the
+    // end (4096x4096: 4.44 / 4.74 / 5.04 us at 2 / 3 / 4 rows against 4.55 / 4.83 / 5.19 through
+    // the loop).  A three-unit path lost 5 % to the loop (4096x6144, 2 rows), and in the
+    // single-row kernels, which are held to 80 registers, any extra path made the loop beside it
+    // 4-7 % slower, so those keep the loop for every length.
     if (total == 1) {
       compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
       if constexpr (MULTI) finish_tile<MB>(acc, slot);
+    } else if (MB >= 2 && !MULTI && total == 2) {
+      advance<MULTI>(cur, walk);
+      load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
+      __builtin_amdgcn_sched_barrier(0);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fb, c, short_ok);
     } else {
       // The prefetches are unconditional: past the wave's last unit every weight offset is out
       // of the descriptor's range, the loads return zero without touching memory, and the
