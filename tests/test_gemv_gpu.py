@@ -482,13 +482,16 @@ def test_vocabulary_projection_one_tile_per_workgroup(gpu):
 
 # Shapes on which the remaining launch rules were measured, each with the plan field that shows the
 # rule took effect: whole-k single-wave workgroups, one-unit waves at 5-8 k steps (in and over the
-# usual wave count), matrix cores from 3 rows, the tile count per activation stage and the balanced
+# usual wave count), paired tiles, the four-wave limit of long reductions, matrix cores from 3 rows, the tile count per activation stage and the balanced
 # k split of the LDS-staged kernel.
 RULES = [
     ("whole_k_m1", 13824, 5120, 1, dict(matrix_core=0, threads=64, split_k=1, steps_per_wave=10)),
     ("whole_k_m2", 13824, 5120, 2, dict(matrix_core=0, threads=64, split_k=1)),
     ("one_unit_waves_m2", 6144, 4096, 2, dict(matrix_core=0, split_k=8, steps_per_wave=1)),
     ("one_unit_waves_11008_waves", 22016, 4096, 1, dict(matrix_core=0, split_k=8, workgroups=1376)),
+    ("paired_tiles", 5120, 5120, 1, dict(matrix_core=0, tiles_per_wg=2, split_k=2, workgroups=160)),
+    ("paired_tiles_m2_long_k", 7168, 14336, 2, dict(matrix_core=0, tiles_per_wg=2, split_k=2, steps_per_wave=14)),
+    ("four_waves_from_16_k_steps", 9216, 8192, 1, dict(matrix_core=0, tiles_per_wg=1, split_k=4, steps_per_wave=4)),
     ("matrix_cores_at_3_rows", 5120, 4096, 3, dict(matrix_core=2)),
     ("two_tiles_even_split", 5120, 5120, 8, dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=5)),
     ("two_tiles_592_workgroups", 18944, 3584, 8, dict(matrix_core=2, tiles_per_wg=2, workgroups=592)),
