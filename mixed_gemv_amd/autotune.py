@@ -51,8 +51,10 @@ class _Problem:
     """Synthetic operands of one problem, resident in device memory.  Any byte string is a valid
     preprocessed weight buffer, so the weights are random bytes."""
 
-    def __init__(self, n_out, k, weight_bits, quant_op, group_size, m_batch, bias, device, seed, cold_bytes):
+    def __init__(self, n_out, k, weight_bits, quant_op, group_size, m_batch, bias, device, seed, cold_bytes,
+                 element="f16"):
         import torch
+        dtype = torch.bfloat16 if element == "bf16" else torch.half
         self.args = (n_out, m_batch, k, group_size, int(quant_op), weight_bits)
         qt = api.QuantType.W4_A16 if weight_bits == 4 else api.QuantType.W8_A16
         w_bytes = api.preprocessed_size((k, n_out), qt)
@@ -61,11 +63,11 @@ class _Problem:
         self.sets = max(4, -(-cold_bytes // per_set) + 1)
         gen = torch.Generator(device=device).manual_seed(seed)
         self.w = torch.randint(0, 256, (self.sets, w_bytes), dtype=torch.uint8, device=device, generator=gen)
-        self.s = (torch.rand((self.sets, groups, n_out), device=device, generator=gen) * 0.019 + 0.001).half()
-        self.z = (torch.rand((self.sets, groups, n_out), device=device, generator=gen) * 0.1 - 0.05).half()
-        self.x = (torch.rand((m_batch, k), device=device, generator=gen) * 2 - 1).half()
-        self.bias = (torch.rand((n_out,), device=device, generator=gen) * 0.2 - 0.1).half() if bias else None
-        self.y = torch.empty((m_batch, n_out), dtype=torch.half, device=device)
+        self.s = (torch.rand((self.sets, groups, n_out), device=device, generator=gen) * 0.019 + 0.001).to(dtype)
+        self.z = (torch.rand((self.sets, groups, n_out), device=device, generator=gen) * 0.1 - 0.05).to(dtype)
+        self.x = (torch.rand((m_batch, k), device=device, generator=gen) * 2 - 1).to(dtype)
+        self.bias = (torch.rand((n_out,), device=device, generator=gen) * 0.2 - 0.1).to(dtype) if bias else None
+        self.y = torch.empty((m_batch, n_out), dtype=dtype, device=device)
 
     def launch(self, i):
         n_out, m_batch, k, group_size, quant_op, bits = self.args
@@ -114,12 +116,13 @@ def install(entry):
 
 def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, group_size=128,
          m_batch=1, bias=False, device="cuda:0", launches=400, rounds=2, min_gain=0.02, seed=1,
-         cold_bytes=_CACHE_BYTES, log=None):
+         cold_bytes=_CACHE_BYTES, log=None, element="f16"):
     """Measures the candidate plans for this problem and installs the fastest, unless it beats the
     built-in plan by less than `min_gain` (then the table is left alone for this key).  Returns a
     dict with the chosen entry (or None), the built-in time and every measurement.  `cold_bytes`
     is how much operand data is rotated between two uses of the same buffers (default: more than
-    the Infinity Cache).
+    the Infinity Cache).  `element` ("f16" / "bf16") picks the entry points that are timed; the table
+    itself is shared by both, so tune for the element type the process will run.
 
     Must not run while other threads launch GEMVs: the candidates are applied through the
     process-wide overrides."""
@@ -129,7 +132,7 @@ def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCA
     device = torch.device(device)
     key = _key(n_out, k, weight_bits, quant_op, group_size, m_batch)
     prob = _Problem(n_out, k, weight_bits, api.WeightOnlyQuantOp(quant_op), key[3], m_batch, bias, device, seed,
-                    cold_bytes)
+                    cold_bytes, element)
     seen, results = {}, []
     try:
         with torch.cuda.device(device):
@@ -139,7 +142,7 @@ def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCA
                 prob.time_us(launches)
             for cand in candidate_plans(n_out, k, weight_bits, m_batch):
                 _apply(cand)
-                geometry = tuple(sorted(api.query_launch(n_out, m_batch, k, weight_bits, key[3]).items()))
+                geometry = tuple(sorted(api.query_launch(n_out, m_batch, k, weight_bits, key[3], element=element).items()))
                 if geometry in seen:
                     continue
                 seen[geometry] = cand

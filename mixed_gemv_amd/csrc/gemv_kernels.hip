@@ -292,7 +292,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // 10.3 at 5 waves per tile; 27648x5120: 15.6 against 17.5 at 3; 14848x6144: 10.6 against 12.1
     // at 6; 13824x8192: 12.6 against 13.7 at 8).  With a worse fit they lose (17408x5120, 1088
     // tiles: 13.8 against 12.4), and the halving below stands.
-    const bool whole_k_waves = !mc && m_batch <= 2 && (long long)groups * split_k > kWaveBudget &&
+    const bool whole_k_waves = !mc && !knobs.wide_waves && m_batch <= 2 && (long long)groups * split_k > kWaveBudget &&
                                (long long)tiles * 100 >= (long long)ceil_div(tiles, kSimds) * kSimds * 80;
     if (whole_k_waves) split_k = 1;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
@@ -303,6 +303,9 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // ones (9216x14336: 16.9 us against 18.1 at 7 waves; 10240x11008: 14.8 against 15.3 at 11;
     // 10240x8192 and 11008x8192: level).
     if (!mc && ksteps >= 16 && split_k > 4) split_k = 4;
+    // The bfloat16 kernels are bound by their arithmetic, and two-unit waves are their worst
+    // length by far (13824x5120: 18.9 us at 5 waves of 2 units against 14.0 at 2 waves of 5).
+    if (knobs.wide_waves && !mc && split_k > 1 && ceil_div(ksteps, split_k) == 2) split_k = (split_k + 1) / 2;
   }
   int tiles_per_wg = pair_tiles ? 2 : 1;
   int workgroup_cap = 0;
@@ -313,9 +316,12 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // The four waves are tw tile sequences x 4/tw k-split waves, tw as large as still fits evenly.
     // Walks of more than 7 tiles lose to one tile per workgroup (128256x4096, 8 tiles per wave:
     // 51.5 us against 47.3; 151936x2048, 19 tiles: 31.9 against 29.8), so those are left out.
+    // (The bfloat16 kernels want every SIMD busy more than they want equal walks: 28672x8192 takes
+    // 35.5 us with one tile and four waves per workgroup against 38.4 with walks of 7 tiles.)
+    const int longest_walk = knobs.wide_waves ? 1 : 7;
     for (int tw = 4; tw >= 1; tw /= 2) {
       const int sequences = kNumCus * tw;
-      if (ceil_div(tiles, sequences) > 7) continue;
+      if (ceil_div(tiles, sequences) > longest_walk) continue;
       if ((long long)ceil_div(tiles, sequences) * sequences * 100 <= (long long)tiles * 103) {
         tiles_per_wg = tw;
         split_k = 4 / tw;
