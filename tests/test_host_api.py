@@ -371,3 +371,19 @@ def test_builtin_launch_rules_on_the_shapes_they_were_measured_on(shape, want):
     assert got["threads"] <= 1024 and got["threads"] % 64 == 0
     per_workgroup = got["tiles_per_wg"] * got["tiles_per_wave"] * got["tiles_in_sequence"]
     assert got["workgroups"] * per_workgroup >= tiles
+
+
+def test_bf16_launch_rules_differ_where_they_were_measured_to():
+    """The bfloat16 kernels are bound by arithmetic: no tile walks, no whole-k single-wave workgroups,
+    no two-unit waves; at most 8 waves per workgroup."""
+    q = lambda n, m, k: mg.query_launch(n, m, k, 4, 128, element="bf16")
+    c5 = q(28672, 1, 8192)
+    assert (c5["workgroups"], c5["split_k"], c5["tiles_in_sequence"]) == (1792, 4, 1), c5
+    assert mg.query_launch(28672, 1, 8192, 4, 128)["tiles_in_sequence"] == 7       # fp16 walks 7 tiles
+    mlp = q(13824, 1, 5120)
+    assert mlp["split_k"] > 1 and mlp["steps_per_wave"] != 2, mlp
+    assert mg.query_launch(13824, 1, 5120, 4, 128)["split_k"] == 1                 # fp16: whole-k waves
+    assert q(8192, 1, 8192)["workgroups"] == 256                                   # one tile per sequence: kept
+    for n, m, k in [(4096, 1, 4096), (1024, 1, 8192), (22016, 1, 4096), (5120, 2, 5120), (4096, 16, 4096)]:
+        assert q(n, m, k)["threads"] <= 512, (n, m, k)
+        assert q(n, m, k)["matrix_core"] in (0, 2)                                 # no register-operand kernel for bf16
