@@ -42,7 +42,7 @@ WORKLOADS = {
            "int4 group-64 scale+zero GEMV + bias, N=K=8192"),
     "c5": (28672, 8192, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
            "int4 group-128 scale+zero GEMV, M=1, K=8192, N=28672"),
-    # not a BASELINE config: a vocabulary projection, the longest launch a decoder step has
+    # not one of the benchmark configurations: a vocabulary projection, the longest launch a decoder step has
     "vocab": (128256, 4096, 4, 3, 128, 1, False, "normal", (0.001, 0.02),
               "int4 group-128 scale+zero GEMV, M=1, K=4096, N=128256 (vocabulary projection)"),
 }

@@ -437,7 +437,7 @@ def test_adaptor_mirror_runs(gpu):
 
 
 FULL = [
-    # BASELINE configurations at their real sizes
+    # the benchmark configurations at their real sizes
     ("c1_int8_percol", 4096, 4096, 8, PER_COLUMN, 0, 1, True, "uniform", (0.001, 0.01)),
     ("c2_int4_g128_scale", 4096, 4096, 4, SCALE_ONLY, 128, 1, True, "uniform", (0.001, 0.02)),
     ("ns_int4_g128_sz", 4096, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "uniform", (0.001, 0.02)),
