@@ -179,9 +179,8 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Which of the two matrix-core kernels serves the small batches:
- *   MGEMV_MATRIX_CORE_AUTO (default)          the register-operand kernel, one tile per wave, on matrices
- *                                             of up to 256 16-row tiles with up to 5 activation rows or
- *                                             a reduction of up to 4 k steps, else the LDS-staged kernel;
+ *   MGEMV_MATRIX_CORE_AUTO (default)          the LDS-staged kernel wherever the matrix has at least two
+ *                                             16-row tiles, else the register-operand kernel;
  *   MGEMV_MATRIX_CORE_REGISTER_OPERAND        always the kernel that reads its activation operand from
  *                                             L2 into registers;
  *   MGEMV_MATRIX_CORE_LDS_STAGED              the LDS-staged kernel wherever the matrix has at least two

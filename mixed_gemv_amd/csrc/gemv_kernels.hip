@@ -174,16 +174,13 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
   const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch);
-  // Small problems (up to 256 tiles) with few rows or a short reduction take the register-operand
-  // kernel with one tile per wave: a lane of a row past m_batch loads nothing there, and no barrier
-  // ties the waves of a workgroup together (1024x2048, 5 rows: 3.4 us against 4.6 us LDS-staged;
-  // 2048x2048, 6 rows: 3.7 against 3.8; 1024x2048, 16 rows: 4.4 against 4.9).  With a longer
-  // reduction the LDS-staged kernel with one tile per workgroup is level at 5 rows and ahead from 6
-  // (4096x4096: 5.4 against 5.6 at 6 rows, 5.4 against 6.1 at 8; 2048x8192, 6 rows: 7.5 against 7.9),
-  // and so it is from 384 tiles at any row count.
-  const bool small_problem = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && tiles <= 256 &&
-                             (m_batch <= 5 || ksteps <= 4);
-  if (mc && knobs.matrix_core_variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND && !small_problem && tiles >= 2) {
+  // The LDS-staged kernel serves every matrix-core launch of two or more tiles.  (While its loop
+  // still had a workgroup barrier per k step, the register-operand kernel was ahead on problems of
+  // up to 256 tiles with up to 5 rows or up to 4 k steps; without the barrier the LDS-staged kernel
+  // with one tile per workgroup wins there too -- 4096x4096, 5 rows: 4.98 us against 5.34;
+  // 2048x8192, 5 rows: 6.5 against 7.5; 2048x2048, 8 rows: 3.68 against 3.91 -- or is level,
+  // 2048x2048, 5 rows: 3.62 against 3.57.)
+  if (mc && knobs.matrix_core_variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND && tiles >= 2) {
     // LDS-staged kernel: the tiles of a workgroup share the activation stage; k split as long as
     // the launch stays within 2048 waves (measured: 8192x8192 best at 4 k-split waves, 11008x4096
     // at 2, 28672x8192 at 1).
@@ -243,7 +240,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   // T = 1 at 8-16 activation rows; T = 4 leaves too few waves to cover the load latency.
   int tiles_per_wave = 1;
   if (mc) {
-    tiles_per_wave = tiles >= 256 && !small_problem ? 2 : 1;
+    tiles_per_wave = tiles >= 256 ? 2 : 1;
     if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
   }
   const int groups = ceil_div(tiles, tiles_per_wave);

@@ -166,7 +166,7 @@ def test_launch_query_knows_the_bf16_kernels(gpu):
     # 8-wave workgroups at most, and only the LDS-staged matrix-core kernel
     assert mg.query_launch(1024, 1, 8192, 4, 128)["threads"] == 1024
     assert mg.query_launch(1024, 1, 8192, 4, 128, element="bf16")["threads"] == 512
-    assert mg.query_launch(1024, 5, 2048, 4, 128)["matrix_core"] == 1
+    assert mg.query_launch(16, 7, 512, 4, 128)["matrix_core"] == 1                      # fp16, a single tile: register operand
     assert mg.query_launch(1024, 5, 2048, 4, 128, element="bf16")["matrix_core"] == 2
     assert mg.query_launch(16, 7, 512, 4, 128, element="bf16")["matrix_core"] == 0      # a single tile
 

@@ -332,9 +332,8 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     dev = DeviceProblem(prob, gpu)
     y_all = dev.run().copy()
     assert np.array_equal(y_all.view(np.uint16), dev.run().view(np.uint16))
-    assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (0 if m_batch < 5 else 1)   # few tiles, short k: register operand
-    assert mg.query_launch(80, m_batch, 4096, 4)["matrix_core"] == (0 if m_batch < 5 else 1 if m_batch <= 5 else 2)
-    assert mg.query_launch(80, 7, 2048, 4)["matrix_core"] == 1   # few tiles, <= 8 rows: register operand
+    assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (0 if m_batch < 5 else 2)   # LDS-staged from 2 tiles
+    assert mg.query_launch(16, 7, 2048, 4)["matrix_core"] == 1    # a single tile: register operand
     assert mg.query_launch(8192, 7, 2048, 4)["matrix_core"] == 2
     single = Problem("rows", 80, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True)
     for b in range(m_batch):
@@ -522,11 +521,11 @@ def test_hip_graph_replays_match_eager_launches(gpu):
     results bit for bit, with eager work and synchronisations between the replays."""
     import torch
     probs = [Problem("g_valu", 320, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=2, bias=True),
-             Problem("g_reg", 320, 2048, 4, SCALE_AND_ZEROS, 64, m_batch=6, bias=True),      # register-operand matrix core
+             Problem("g_reg", 16, 2048, 4, SCALE_AND_ZEROS, 64, m_batch=6, bias=True),       # one tile: register-operand matrix core
              Problem("g_lds", 320, 2048, 8, PER_COLUMN, 0, m_batch=16, bias=False),          # LDS-staged, 16 rows staged
              Problem("g_bf16", 320, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True, element="bf16")]
     devs = [DeviceProblem(p, gpu) for p in probs]
-    assert [mg.query_launch(320, p.m_batch, 2048, p.bits)["matrix_core"] for p in probs[:3]] == [0, 1, 2]
+    assert [mg.query_launch(p.n_out, p.m_batch, 2048, p.bits)["matrix_core"] for p in probs[:3]] == [0, 1, 2]
     eager = [d.run().copy() for d in devs]
 
     def launch_all():

@@ -338,7 +338,8 @@ BUILTIN_PLANS = [
     ((17408, 1, 5120), dict(matrix_core=0, workgroups=1088, split_k=5, steps_per_wave=2)),
     # matrix cores: from 5 rows anywhere, from 3 rows on more than 256 tiles, from 2 rows on many tiles
     ((4096, 4, 4096), dict(matrix_core=0)),
-    ((4096, 5, 4096), dict(matrix_core=1)),
+    ((4096, 5, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
+    ((16, 8, 4096), dict(matrix_core=1)),                      # a single tile: the register-operand kernel
     ((4096, 8, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
     ((5120, 3, 4096), dict(matrix_core=2)),
     ((4096, 4, 14336), dict(matrix_core=0)),
