@@ -163,7 +163,11 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced) {
   if (forced > 0) return m_batch >= forced;
   const long long units = (long long)tiles * ksteps;
+  // 4 rows on 129-256 tiles: the barrier-free one-tile matrix-core launch is ahead from 16 k steps
+  // (4096x8192: 6.9 us against 7.4; 4096x14336: 9.7 against 10.7; 3584x18944: 12.3 against 13.8)
+  // and level below (4096x4096: 5.07 against 5.00); 2 and 3 rows stay on the VALU kernel there.
   return m_batch >= 5 || (m_batch >= 3 && tiles > kNumCus && units >= 2048) ||
+         (m_batch >= 4 && tiles > kNumCus / 2 && ksteps >= 16) ||
          (m_batch >= 2 && tiles >= 1536 && (ksteps >= 8 || units > 16384));
 }
 

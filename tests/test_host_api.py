@@ -342,7 +342,9 @@ BUILTIN_PLANS = [
     ((16, 8, 4096), dict(matrix_core=1)),                      # a single tile: the register-operand kernel
     ((4096, 8, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
     ((5120, 3, 4096), dict(matrix_core=2)),
-    ((4096, 4, 14336), dict(matrix_core=0)),
+    ((4096, 3, 14336), dict(matrix_core=0)),
+    ((4096, 4, 14336), dict(matrix_core=2, tiles_per_wg=1)),   # 4 rows, 129-256 tiles, from 16 k steps
+    ((2048, 4, 8192), dict(matrix_core=0)),
     ((10240, 2, 8192), dict(matrix_core=0)),
     ((28672, 2, 8192), dict(matrix_core=2)),
     ((50304, 2, 2048), dict(matrix_core=0)),
