@@ -160,7 +160,7 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 // against 16.4; 28672x8192: 25.9 against 27.3; 10240x8192: 14.2 against 12.7 the other way), and
 // with fewer than 8 k steps only when one-unit VALU waves would not fit the machine (50304x2048,
 // 12576 units: 15.2 against 12.8 the other way; 151936x2048, 37984 units: 33.1 against 35.1).
-inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced) {
+inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, bool bf16) {
   if (forced > 0) return m_batch >= forced;
   const long long units = (long long)tiles * ksteps;
   // 4 rows on 129-256 tiles: the barrier-free one-tile matrix-core launch is ahead from 16 k steps
@@ -168,7 +168,7 @@ inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced) {
   // and level below (4096x4096: 5.07 against 5.00); 2 and 3 rows stay on the VALU kernel there.
   return m_batch >= 5 || (m_batch >= 3 && tiles > kNumCus && units >= 2048) ||
          (m_batch >= 4 && tiles > kNumCus / 2 && ksteps >= 16) ||
-         (m_batch >= 2 && tiles >= 1536 && (ksteps >= 8 || units > 16384));
+         (m_batch >= 2 && !bf16 && tiles >= 1536 && (ksteps >= 8 || units > 16384));  // bf16, 28672x8192, 2 rows: 40.6 us against 37.8
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -177,7 +177,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
-  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch);
+  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves);
   // The LDS-staged kernel serves every matrix-core launch of two or more tiles.  (While its loop
   // still had a workgroup barrier per k step, the register-operand kernel was ahead on problems of
   // up to 256 tiles with up to 5 rows or up to 4 k steps; without the barrier the LDS-staged kernel

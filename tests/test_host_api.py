@@ -386,6 +386,7 @@ def test_bf16_launch_rules_differ_where_they_were_measured_to():
     mlp = q(13824, 1, 5120)
     assert mlp["split_k"] > 1 and mlp["steps_per_wave"] != 2, mlp
     assert mg.query_launch(13824, 1, 5120, 4, 128)["split_k"] == 1                 # fp16: whole-k waves
+    assert q(28672, 2, 8192)["matrix_core"] == 0 and q(28672, 3, 8192)["matrix_core"] == 2   # 2 rows stay on the VALU kernel
     assert q(8192, 1, 8192)["workgroups"] == 256                                   # one tile per sequence: kept
     for n, m, k in [(4096, 1, 4096), (1024, 1, 8192), (22016, 1, 4096), (5120, 2, 5120), (4096, 16, 4096)]:
         assert q(n, m, k)["threads"] <= 512, (n, m, k)
