@@ -176,7 +176,8 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
 /* Smallest m_batch served by the matrix-core kernels instead of the VALU kernel.  0 restores the
  * built-in rule (from 5 rows; from 3 rows on matrices of more than 256 16-row tiles, n_out > 4096; from 4 rows
  * on more than 128 tiles with 16 or more k steps;
- * from 2 rows on 1536 or more tiles with 8 or more k steps or more than 16384 units; never for a single row); 17 keeps every batch size on the VALU kernel.  For tuning and tests.  Process-wide. */
+ * from 2 rows on 1536 or more tiles with 8 or more k steps or more than 16384 units; int8 weights: from 5 rows,
+ * from 3 rows on 1536 or more tiles; never for a single row); 17 keeps every batch size on the VALU kernel.  For tuning and tests.  Process-wide. */
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Which of the two matrix-core kernels serves the small batches:

@@ -160,8 +160,12 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 // against 16.4; 28672x8192: 25.9 against 27.3; 10240x8192: 14.2 against 12.7 the other way), and
 // with fewer than 8 k steps only when one-unit VALU waves would not fit the machine (50304x2048,
 // 12576 units: 15.2 against 12.8 the other way; 151936x2048, 37984 units: 33.1 against 35.1).
-inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, bool bf16) {
+inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, bool bf16, int bits) {
   if (forced > 0) return m_batch >= forced;
+  // int8 weights: twice the bytes per VALU instruction, so the VALU kernel holds out longer --
+  // ahead at 2-4 rows on every shape measured (8192x8192, 3 rows: 13.0 us against 14.8; 4096x11008,
+  // 4 rows: 10.4 against 11.5) except the largest (28672x8192, 3 rows: 41.4 against 39.7).
+  if (bits == 8) return m_batch >= 5 || (m_batch >= 3 && tiles >= 1536);
   const long long units = (long long)tiles * ksteps;
   // 4 rows on 129-256 tiles: the barrier-free one-tile matrix-core launch is ahead from 16 k steps
   // (4096x8192: 6.9 us against 7.4; 4096x14336: 9.7 against 10.7; 3584x18944: 12.3 against 13.8)
@@ -177,7 +181,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
-  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves);
+  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves, bits);
   // The LDS-staged kernel serves every matrix-core launch of two or more tiles.  (While its loop
   // still had a workgroup barrier per k step, the register-operand kernel was ahead on problems of
   // up to 256 tiles with up to 5 rows or up to 4 k steps; without the barrier the LDS-staged kernel

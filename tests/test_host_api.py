@@ -391,3 +391,10 @@ def test_bf16_launch_rules_differ_where_they_were_measured_to():
     for n, m, k in [(4096, 1, 4096), (1024, 1, 8192), (22016, 1, 4096), (5120, 2, 5120), (4096, 16, 4096)]:
         assert q(n, m, k)["threads"] <= 512, (n, m, k)
         assert q(n, m, k)["matrix_core"] in (0, 2)                                 # no register-operand kernel for bf16
+
+
+def test_int8_weights_keep_two_to_four_rows_on_the_valu_kernel():
+    q = lambda n, m, k: mg.query_launch(n, m, k, 8, 128)["matrix_core"]
+    assert [q(8192, m, 8192) for m in (2, 3, 4, 5)] == [0, 0, 0, 2]
+    assert [q(4096, m, 11008) for m in (3, 4, 5)] == [0, 0, 2]
+    assert [q(28672, m, 8192) for m in (2, 3, 4)] == [0, 2, 2]
