@@ -42,16 +42,22 @@ typedef enum mgemv_status {
   MGEMV_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
   MGEMV_ERR_RANK = 2,           /* shape rank not 2 or 3 (utils/preprocess.h:486-489) */
   MGEMV_ERR_ROWS = 3,           /* n_out not a multiple of 4 (utils/preprocess.h:319-322) */
-  MGEMV_ERR_COLS = 4,           /* k not a multiple of the 128-bit access (utils/preprocess.h:324-327) */
+  MGEMV_ERR_COLS = 4,           /* k not a multiple of 8 (utils/preprocess.h:324-327) */
   MGEMV_ERR_GROUP_SIZE = 5,     /* group_size < 64 (gemv/device/gemv_adaptor.h:199-203), not a multiple of 32, or not dividing k */
   MGEMV_ERR_QUANT_OP = 6,       /* quant_op not 1, 2 or 3 (gemv/weight_only_quant_op.h:12-18) */
   MGEMV_ERR_QUANT_TYPE = 7,     /* weight type not W8_A16 / W4_A16 (utils/preprocess.h:110, 287-288) */
   MGEMV_ERR_BATCH = 8,          /* batch_count < 1 or m_batch outside [1, MGEMV_MAX_M_BATCH] */
-  MGEMV_ERR_LAYOUT = 9,         /* layout flag not row/column major, or a row-major transpose whose dims are not multiples of 64 elements (utils/preprocess.h:157-162) */
+  MGEMV_ERR_LAYOUT = 9,         /* layout flag not row/column major (utils/preprocess.h:486-489; the reference's further
+                                   demand that a row-major matrix have dimensions of whole 64-element tiles,
+                                   utils/preprocess.h:157-162, does not apply: any legal n_out, k is transposed) */
   MGEMV_ERR_SIZE = 10,          /* a dimension is <= 0 or overflows the 32-bit index space of the kernels */
   MGEMV_ERR_LAUNCH = 11,        /* the HIP runtime refused the launch (gemv/device/gemv_adaptor.h:249-254) */
-  MGEMV_ERR_NO_DEVICE = 12,     /* no usable gfx950 device */
-  MGEMV_ERR_ALIGNMENT = 13      /* a device pointer is not aligned as required (16 B weights/activations, 4 B scales) */
+  MGEMV_ERR_NO_DEVICE = 12,     /* the stream's device (the current device for the null stream) is not a gfx950 */
+  MGEMV_ERR_ALIGNMENT = 13,     /* a device pointer is not aligned as required: weights and activations 16 bytes (and
+                                   the batch strides to match); scales, zeros, bias, outputs 2 bytes; the output of
+                                   mgemv_dequantize 4 bytes */
+  MGEMV_ERR_LEADING_DIMENSION = 14, /* mgemv_gemv_arguments: a leading dimension other than the dense one */
+  MGEMV_ERR_ALLOCATION = 15     /* mgemv_host_gemv: device memory could not be allocated */
 } mgemv_status;
 
 /* gemv/weight_only_quant_op.h:12-18 — same numeric values. */
@@ -80,7 +86,8 @@ MGEMV_API int mgemv_version(void);
  * ---------------------------------------------------------------------------------------- */
 
 /* Replaces SubBytePacker<int4b_t,int8_t>::pack (utils/preprocess.h:55-84).
- * Packs n_unpacked (even) signed 4-bit values held one per int8 into n_unpacked/2 bytes:
+ * Packs n_unpacked signed 4-bit values held one per int8 into n_unpacked/2 bytes (an odd
+ * n_unpacked is MGEMV_ERR_SIZE):
  * element 2i in bits 0..3 of byte i, element 2i+1 in bits 4..7.  Values are truncated to
  * their low 4 bits, as in the reference. */
 MGEMV_API int mgemv_pack_int4(uint8_t *packed, const int8_t *unpacked, size_t n_unpacked);
@@ -156,6 +163,50 @@ MGEMV_API int mgemv_gemv_batched(const void *weights, const uint16_t *x, const u
                                  int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
                                  int64_t stride_bias, int64_t stride_y, void *stream);
 
+/* GemvAdaptor::Arguments (gemv/device/gemv_adaptor.h:114-178) as a plain struct, and
+ * GemvAdaptor::operator()(args, stream) (:258-261) as one call: everything mgemv_gemv_batched
+ * takes, plus the epilogue's alpha and beta and the leading dimensions of the reference's
+ * TensorRefs.  y = element( alpha * acc + beta * bias ), computed in fp32 with the outer
+ * multiply-add fused (the reference's LinearCombination, mixed_gemv_test.cu:72-81;
+ * epilogue/threadblock/epilogue.h:64, 93); bias == NULL drops the term.  alpha = beta = 1 is
+ * mgemv_gemv_batched bit for bit.  The operands are dense: a leading dimension must be 0
+ * ("dense") or the value the reference's caller passes for that operand -- lda 4*k (or k), ldb k
+ * (0 is also accepted for m_batch == 1, mixed_gemv_test.cu:137), ld_scale / ld_zero / ldc / ldd
+ * n_out (mixed_gemv_test.cu:136-140, 153-154) -- anything else is MGEMV_ERR_LEADING_DIMENSION,
+ * never a silently different result.  Batch strides as in mgemv_gemv_batched. */
+enum { MGEMV_ELEMENT_F16 = 0, MGEMV_ELEMENT_BF16 = 1 };
+typedef struct mgemv_arguments {
+  int n_out, m_batch, k;                    /* problem_size: the reference's (M, N, K) */
+  const void *weights; int64_t lda;         /* ref_A: preprocessed weights */
+  const uint16_t *x; int64_t ldb;           /* ref_B */
+  const uint16_t *scale; int64_t ld_scale;  /* ref_scale */
+  const uint16_t *zero_add; int64_t ld_zero;/* ref_zero_point: the folded additive term */
+  const uint16_t *bias; int64_t ldc;        /* ref_C */
+  uint16_t *y; int64_t ldd;                 /* ref_D */
+  float alpha, beta;                        /* epilogue */
+  int group_size, batch_count;
+  int64_t batch_stride_weights, batch_stride_x, batch_stride_scale, batch_stride_bias, batch_stride_y;
+  int quant_op, weight_bits;                /* template parameters in the reference */
+  int element;                              /* MGEMV_ELEMENT_F16 / _BF16: ElementB = ElementScale = ElementOutput */
+} mgemv_arguments;
+MGEMV_API int mgemv_gemv_arguments(const mgemv_arguments *args, void *stream);
+
+/* host::reference::MixedGemv::operator() (host/mixed_gemv.h:60-70) with the GPU behind it: the
+ * same argument list and meaning -- HOST pointers, `weights` the UN-preprocessed quantised
+ * matrix ([n_out][k] row-major; int4 packed two per byte as utils/vector_subbyte.h:150-156 lays
+ * them out, or int8), `zero_point` the int8 zero points [k/group_size][n_out] (not folded; read
+ * only in mode 3), `bias` may be NULL -- so a caller of the reference's HOST_CHECK path can be
+ * pointed at the device without touching its data.  Preprocesses, folds the zero points
+ * (utils/preprocess.h:94-101), uploads, runs mgemv_gemv on the null stream of the current
+ * device and downloads; synchronous.  Unlike every other device entry point it ALLOCATES (one
+ * hipMalloc / hipFree per call): a convenience and parity entry, not a hot path.  Beyond the
+ * reference (which exits unless N == 1, :72-75) m_batch up to 16 rows is accepted; batch must be
+ * 1 (:77-80).  quant_op and weight_bits are template parameters in the reference, which only
+ * instantiates int4 with zero points (:23-42). */
+MGEMV_API int mgemv_host_gemv(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t *weights,
+                              const uint16_t *x, const uint16_t *scale, const int8_t *zero_point,
+                              const uint16_t *bias, uint16_t *y, int quant_op, int weight_bits);
+
 /* Parity/debug entry: writes the dequantised weights, fp16 [n_out][k] row-major, produced by
  * the SAME device conversion and dequantisation code the GEMV kernels use
  * (gemv/interleaved_numeric_conversion.h:62-81, 232-291 then gemv/warp/warp_dequantizer.h:52-59, 86-92).
@@ -212,7 +263,8 @@ MGEMV_API int mgemv_set_dequant_form(int form);
  * an instantiation the reference itself still rejects at compile time
  * (gemv/threadblock/default_dq_mma_simt.h:133-134).  Dequantisation is a bf16 multiply and a bf16
  * add, each rounded to nearest even; accumulation is fp32; the output is rounded once to bf16.
- * Every m_batch runs on the VALU kernel (groups of 4 activation rows per launch). */
+ * Kernel choice follows the fp16 rules (mgemv_set_matrix_core_threshold), except that of the two
+ * matrix-core kernels only the LDS-staged one exists for bf16 (mgemv_query_launch_bf16 tells). */
 MGEMV_API int mgemv_gemv_bf16(const void *weights, const uint16_t *x, const uint16_t *scale,
                               const uint16_t *zero_add, const uint16_t *bias, uint16_t *y, int n_out, int m_batch,
                               int k, int group_size, int quant_op, int weight_bits, void *stream);
@@ -264,9 +316,15 @@ MGEMV_API int mgemv_tuned_plan_count(void);
  * out[6] = tiles per wave (matrix-core path), out[7] = most tiles a wave walks one after the
  * other (VALU path). */
 MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]);
-/* The same for the _bf16 entry points (their kernels are compiled for at most 8 waves per workgroup, and of
+/* mgemv_query_launch assumes an unpartitioned MI355X (256 compute units); a launch plans for the
+ * compute units of the device its stream belongs to.
+ * The same for the _bf16 entry points (their kernels are compiled for at most 8 waves per workgroup, and of
  * the matrix-core kernels only the LDS-staged one exists for bf16). */
 MGEMV_API int mgemv_query_launch_bf16(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]);
+/* The same for either element type (MGEMV_ELEMENT_*) and a device of num_compute_units compute
+ * units (a partition of an MI355X has 32 per XCD). */
+MGEMV_API int mgemv_query_launch_for(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
+                                     int num_compute_units, int out[8]);
 
 #ifdef __cplusplus
 }

@@ -14,6 +14,8 @@ from .api import (  # noqa: F401
     ZeroPointPreprocessor,
     dequantize,
     device_gemv,
+    gemv_arguments,
+    host_gemv,
     preprocessed_size,
     query_launch,
     set_launch_override,

@@ -154,6 +154,61 @@ def unpreprocess_weights(preprocessed, shape, quant_type=QuantType.W4_A16):
     return dst
 
 
+class _Arguments(ctypes.Structure):
+    """mgemv_arguments (include/mixed_gemv.h)."""
+    _fields_ = [("n_out", ctypes.c_int), ("m_batch", ctypes.c_int), ("k", ctypes.c_int),
+                ("weights", ctypes.c_void_p), ("lda", ctypes.c_int64),
+                ("x", ctypes.c_void_p), ("ldb", ctypes.c_int64),
+                ("scale", ctypes.c_void_p), ("ld_scale", ctypes.c_int64),
+                ("zero_add", ctypes.c_void_p), ("ld_zero", ctypes.c_int64),
+                ("bias", ctypes.c_void_p), ("ldc", ctypes.c_int64),
+                ("y", ctypes.c_void_p), ("ldd", ctypes.c_int64),
+                ("alpha", ctypes.c_float), ("beta", ctypes.c_float),
+                ("group_size", ctypes.c_int), ("batch_count", ctypes.c_int),
+                ("batch_stride_weights", ctypes.c_int64), ("batch_stride_x", ctypes.c_int64),
+                ("batch_stride_scale", ctypes.c_int64), ("batch_stride_bias", ctypes.c_int64),
+                ("batch_stride_y", ctypes.c_int64),
+                ("quant_op", ctypes.c_int), ("weight_bits", ctypes.c_int), ("element", ctypes.c_int)]
+
+
+def gemv_arguments(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, M, N, K, group_size, quant_op, weight_bits=4,
+                   alpha=1.0, beta=1.0, leading_dims=None, batch_count=1, batch_strides=None, stream=None, element=None):
+    """GemvAdaptor::Arguments + operator() in one call (mgemv_gemv_arguments): the epilogue's alpha and
+    beta, and the reference's leading dimensions (lda, ldb, ld_scale, ld_zero, ldc, ldd; None = dense)."""
+    lda, ldb, lds, ldz, ldc, ldd = leading_dims or (0, int(K) if int(N) > 1 else 0, 0, 0, 0, 0)
+    sa, sb, ss, sc, sd = batch_strides or (0, 0, 0, 0, 0)
+    val = lambda p: _dev_ptr(p).value  # noqa: E731
+    a = _Arguments(int(M), int(N), int(K), val(ptr_A), int(lda), val(ptr_B), int(ldb), val(ptr_scale), int(lds),
+                   val(ptr_zero_point), int(ldz), val(ptr_C), int(ldc), val(ptr_D), int(ldd), float(alpha), float(beta),
+                   int(group_size), int(batch_count), int(sa), int(sb), int(ss), int(sc), int(sd), int(quant_op),
+                   int(weight_bits), 1 if _is_bf16(element, ptr_B) else 0)
+    _lib.check(_lib.lib().mgemv_gemv_arguments(ctypes.byref(a), _stream_ptr(stream)), "gemv_arguments")
+
+
+def host_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, B, M, N, K, group_size,
+              quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4):
+    """host_gemv of mixed_gemv_test.cu:167-181, i.e. host::reference::MixedGemv::operator()
+    (host/mixed_gemv.h:60-70), with the GPU behind it: numpy arrays in host memory, UN-preprocessed
+    packed weights [M][K], int8 zero points [K/group_size][M] (mode 3), optional fp16 bias.  Returns
+    the fp16 result [N][M].  There is no CPU path: without a gfx950 device this raises."""
+    w = np.ascontiguousarray(ptr_A).reshape(-1).view(np.uint8)
+    x = np.ascontiguousarray(ptr_B, dtype=np.float16)
+    s = np.ascontiguousarray(ptr_scale, dtype=np.float16)
+    z = None if ptr_zero_point is None else np.ascontiguousarray(ptr_zero_point, dtype=np.int8)
+    b = None if ptr_C is None else np.ascontiguousarray(ptr_C, dtype=np.float16)
+    need = int(M) * int(K) * int(weight_bits) // 8
+    if w.size < need or x.size < int(N) * int(K):
+        raise ValueError("operand smaller than the problem")
+    y = np.empty((int(N), int(M)), dtype=np.float16)
+    null = ctypes.c_void_p(0)
+    st = _lib.lib().mgemv_host_gemv(int(B), int(M), int(N), int(K), int(group_size), _host_ptr(w), _host_ptr(x),
+                                    _host_ptr(s), _host_ptr(z) if z is not None else null,
+                                    _host_ptr(b) if b is not None else null, _host_ptr(y), int(quant_op),
+                                    int(weight_bits))
+    _lib.check(st, "host_gemv")
+    return y
+
+
 def device_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, B, M, N, K, group_size,
                 quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, stream=None,
                 batch_strides=None, element=None):
@@ -257,13 +312,19 @@ def set_dequant_form(form=DEQUANT_AUTO):
     _lib.check(_lib.lib().mgemv_set_dequant_form(int(form)), "set_dequant_form")
 
 
-def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0, element="f16"):
-    """The geometry mgemv_gemv (element="bf16": mgemv_gemv_bf16) would use; group_size as passed to the GEMV
-    (it only selects tuned plans)."""
+def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0, element="f16", num_compute_units=None):
+    """The geometry mgemv_gemv (element="bf16": mgemv_gemv_bf16) would use on an unpartitioned MI355X, or on
+    a device of num_compute_units compute units; group_size as passed to the GEMV (it only selects tuned
+    plans)."""
     out = (ctypes.c_int * 8)()
-    fn = _lib.lib().mgemv_query_launch_bf16 if _is_bf16(element, None) else _lib.lib().mgemv_query_launch
-    _lib.check(fn(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size), ctypes.byref(out)),
-               "query_launch")
+    if num_compute_units is not None:
+        _lib.check(_lib.lib().mgemv_query_launch_for(int(n_out), int(m_batch), int(k), int(weight_bits),
+                                                     int(group_size), 1 if _is_bf16(element, None) else 0,
+                                                     int(num_compute_units), ctypes.byref(out)), "query_launch")
+    else:
+        fn = _lib.lib().mgemv_query_launch_bf16 if _is_bf16(element, None) else _lib.lib().mgemv_query_launch
+        _lib.check(fn(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size), ctypes.byref(out)),
+                   "query_launch")
     keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave",
             "tiles_in_sequence")
     return dict(zip(keys, list(out)))

@@ -267,10 +267,10 @@ __device__ __forceinline__ void store_outputs(const GemvTail& tail, bool has_bia
   if (lane < kTileRows && n < n_out) {
     if constexpr (ACT == kActBf16) {
       const uint16_t* bias = reinterpret_cast<const uint16_t*>(tail.bias);
-      if (has_bias) sum += bf16_low_to_f32(bias[n]);
+      sum = epilogue_value(tail, sum, has_bias, has_bias ? bf16_low_to_f32(bias[n]) : 0.0f);
       reinterpret_cast<uint16_t*>(tail.y)[(size_t)m * (size_t)n_out + n] = (uint16_t)pack_bf16(sum, 0.0f);
     } else {
-      if (has_bias) sum += (float)tail.bias[n];
+      sum = epilogue_value(tail, sum, has_bias, has_bias ? (float)tail.bias[n] : 0.0f);
       tail.y[(size_t)m * (size_t)n_out + n] = (half_t)sum;
     }
   }

@@ -4,9 +4,11 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 #include "kernel_common.h"
 
@@ -65,6 +67,7 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, 
       const uint32_t z_bits = (uint32_t)__builtin_bit_cast(uint16_t, z[i]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        if (k0 + j * G::kWordK >= p.k) continue;  // k is a multiple of 8: whole words
         uint32_t d[kPairs];
         if (take_short) {
           const Bf16Scale bs = make_bf16_scale<BITS, true>(s_bits[i], z_bits);
@@ -82,6 +85,7 @@ __global__ void __launch_bounds__(256) dequantize_kernel(const DequantParams p, 
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      if (k0 + j * G::kWordK >= p.k) continue;  // k is a multiple of 8: whole words
       if constexpr (BITS == 4) {
         half2_t d[4];
         if (take_short) {
@@ -123,6 +127,7 @@ struct PlanKnobs {
   int matrix_core_min_batch = 0;
   int matrix_core_variant = MGEMV_MATRIX_CORE_AUTO;
   bool wide_waves = false;  // the kernel is one of those compiled for at most 8 waves per workgroup
+  int num_cus = kNumCus;    // compute units of the device the launch goes to (256 on an unpartitioned MI355X)
 };
 
 // Tuned plans by problem: (n_out, k, weight bits, group size or 0 for any, m_batch) -> knobs.
@@ -160,28 +165,31 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
 // against 16.4; 28672x8192: 25.9 against 27.3; 10240x8192: 14.2 against 12.7 the other way), and
 // with fewer than 8 k steps only when one-unit VALU waves would not fit the machine (50304x2048,
 // 12576 units: 15.2 against 12.8 the other way; 151936x2048, 37984 units: 33.1 against 35.1).
-inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, bool bf16, int bits) {
+// cus: compute units of the device; the tile and unit counts the rules were measured at (on 256
+// compute units) scale with it.
+inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, bool bf16, int bits, int cus) {
   if (forced > 0) return m_batch >= forced;
   // int8 weights: twice the bytes per VALU instruction, so the VALU kernel holds out longer --
   // ahead at 2-4 rows on every shape measured (8192x8192, 3 rows: 13.0 us against 14.8; 4096x11008,
   // 4 rows: 10.4 against 11.5) except the largest (28672x8192, 3 rows: 41.4 against 39.7).
-  if (bits == 8) return m_batch >= 5 || (m_batch >= 3 && tiles >= 1536);
+  if (bits == 8) return m_batch >= 5 || (m_batch >= 3 && tiles >= 6 * cus);
   const long long units = (long long)tiles * ksteps;
   // 4 rows on 129-256 tiles: the barrier-free one-tile matrix-core launch is ahead from 16 k steps
   // (4096x8192: 6.9 us against 7.4; 4096x14336: 9.7 against 10.7; 3584x18944: 12.3 against 13.8)
   // and level below (4096x4096: 5.07 against 5.00); 2 and 3 rows stay on the VALU kernel there.
-  return m_batch >= 5 || (m_batch >= 3 && tiles > kNumCus && units >= 2048) ||
-         (m_batch >= 4 && tiles > kNumCus / 2 && ksteps >= 16) ||
-         (m_batch >= 2 && !bf16 && tiles >= 1536 && (ksteps >= 8 || units > 16384));  // bf16, 28672x8192, 2 rows: 40.6 us against 37.8
+  return m_batch >= 5 || (m_batch >= 3 && tiles > cus && units >= 8ll * cus) ||
+         (m_batch >= 4 && tiles > cus / 2 && ksteps >= 16) ||
+         (m_batch >= 2 && !bf16 && tiles >= 6 * cus && (ksteps >= 8 || units > 64ll * cus));  // bf16, 28672x8192, 2 rows: 40.6 us against 37.8
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs& knobs) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
+  const int cus = knobs.num_cus > 0 ? knobs.num_cus : cus;  // the thresholds below were measured on 256 and scale with it
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
-  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves, bits);
+  const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves, bits, cus);
   // The LDS-staged kernel serves every matrix-core launch of two or more tiles.  (While its loop
   // still had a workgroup barrier per k step, the register-operand kernel was ahead on problems of
   // up to 256 tiles with up to 5 rows or up to 4 k steps; without the barrier the LDS-staged kernel
@@ -203,17 +211,17 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // against 6.4 at 2; 5120x5120 (320) 7.7 at 2 against 9.3 at 1; 10240x8192 (640) 14.7 at 4
     // against 15.5 at 2; 11008x4096 9.0 at 4 against 9.7 at 2; 28672x8192 27.6 at 4 against 29.5 at 2.
     lp.tiles_per_wg = 1;
-    while (ceil_div(tiles, lp.tiles_per_wg) > kNumCus && lp.tiles_per_wg * 2 <= 8 &&
+    while (ceil_div(tiles, lp.tiles_per_wg) > cus && lp.tiles_per_wg * 2 <= 8 &&
            lp.tiles_per_wg * 4 <= lp.staged_rows)
       lp.tiles_per_wg *= 2;
     // Still more workgroups than compute units: a count just above a multiple of 256 leaves most
     // of the last round idle, and halving the tiles per workgroup evens that out (18944x3584,
     // 8 rows: 296 workgroups of 4 tiles 12.8 us, 592 of 2 tiles 11.8; 22016x4096: 14.4 / 13.3).
     // Largest count whose last round is at least three quarters full.
-    if (ceil_div(tiles, lp.tiles_per_wg) > kNumCus) {
+    if (ceil_div(tiles, lp.tiles_per_wg) > cus) {
       for (int tw = lp.tiles_per_wg; tw >= 1; tw /= 2) {
         const int wgs = ceil_div(tiles, tw);
-        if (wgs * 4 >= ceil_div(wgs, kNumCus) * kNumCus * 3) {
+        if (wgs * 4 >= ceil_div(wgs, cus) * cus * 3) {
           lp.tiles_per_wg = tw;
           break;
         }
@@ -224,7 +232,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
     const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;
-    while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 2048) split *= 2;
+    while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 8 * cus) split *= 2;
     // A split that leaves the last wave nearly idle (10 k steps over 4 waves: 3, 3, 3, 1) loses
     // to half as many evenly loaded waves, as long as the workgroup keeps four (5120x5120, 8 rows,
     // 2 tiles: 7.6 us at 2 waves per tile against 8.1 at 4; 6912x5120, 16 rows: 9.0 against 9.6;
@@ -248,7 +256,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   // T = 1 at 8-16 activation rows; T = 4 leaves too few waves to cover the load latency.
   int tiles_per_wave = 1;
   if (mc) {
-    tiles_per_wave = tiles >= 256 ? 2 : 1;
+    tiles_per_wave = tiles >= cus ? 2 : 1;
     if (ov_t == 1 || ov_t == 2 || ov_t == 4) tiles_per_wave = ov_t;
   }
   const int groups = ceil_div(tiles, tiles_per_wave);
@@ -269,28 +277,28 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   // waves (5120x5120: 5.8 us against 6.2; 6144x8192: 7.7 against 8.3; 5120x14336: 11.0 against
   // 11.5) and one-unit or two-unit waves (7168x8192: 7.8 against 8.7; 6656x11008: 9.9 against
   // 11.3; 7168x14336: 11.8 against 15.3); at 260 tiles they are 1-3 % behind (4160x8192).
-  const bool pair_tiles = !mc && tiles * 8 >= kNumCus * 9 && tiles <= 2 * kNumCus && ksteps >= 9;
+  const bool pair_tiles = !mc && tiles * 8 >= cus * 9 && tiles <= 2 * cus && ksteps >= 9;
   if (pair_tiles) {
-    split_k = tiles <= 384 && ksteps >= 20 ? 4 : 2;
-  } else if (groups <= 384) {
+    split_k = tiles <= cus * 3 / 2 && ksteps >= 20 ? 4 : 2;
+  } else if (groups <= cus * 3 / 2) {
     split_k = ksteps < 4 ? ksteps : 4;
     // With workgroups for at most half the compute units, one unit per wave is 4-5 % ahead up to
     // 16 k steps (1024x4096: 3.38 us against 3.54; 1024x8192: 4.54 against 4.77); with a longer
     // reduction it is not (2048x11008: 6.35 at 8 waves against 6.12).
-    if (!mc && tiles <= 128 && ksteps <= 16) split_k = ksteps;
+    if (!mc && tiles <= cus / 2 && ksteps <= 16) split_k = ksteps;
     // More than one workgroup per compute unit and 5-8 k steps, one or two rows: four waves would take
     // two units each, the one length at which the two-deep pipeline overlaps nothing; one unit
     // per wave is 6-7 % ahead (4608x4096: 4.81 us against 5.13; 6144x4096: 4.98 against 5.29),
     // while at 256 tiles four waves win (4096x4096: 4.08 against 4.33).
-    if (!mc && m_batch <= 2 && tiles > kNumCus && ceil_div(ksteps, 4) == 2) split_k = ksteps;
+    if (!mc && m_batch <= 2 && tiles > cus && ceil_div(ksteps, 4) == 2) split_k = ksteps;
     if (mc) split_k = ksteps < max_waves ? ksteps : max_waves;  // not pipelined: wants waves
   } else {
     // One or two rows and up to 8 k steps: workgroups of up to 8 one-unit waves stay ahead of two-unit
     // waves well past 8192 waves (22016x4096, 11008 waves: 10.9 us against 11.8; 27200x4096,
     // 13600 waves: 12.6 against 13.0; 36864x2560: 11.8 against 12.3).
     const bool short_single_row = !mc && m_batch <= 2 && ksteps <= 8;
-    const int kWaveBudget = short_single_row ? 16384 : 8192;
-    constexpr int kSimds = kNumCus * 4;
+    const int kWaveBudget = (short_single_row ? 64 : 32) * cus;
+    const int kSimds = cus * 4;
     split_k = ksteps < max_waves ? ksteps : max_waves;
     // One wave per unit does not fit the machine at once, and one wave per tile fills at least
     // 80 % of the SIMDs of its last round: the whole-k waves win (13824x5120: 9.1 us against
@@ -302,7 +310,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     if (whole_k_waves) split_k = 1;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
     if (!mc && !short_single_row && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
-        (long long)groups * ((split_k + 1) / 2) >= 4096)
+        (long long)groups * ((split_k + 1) / 2) >= 16 * cus)
       split_k = (split_k + 1) / 2;
     // From 16 k steps four waves with longer pipelines are level with or ahead of more, shorter
     // ones (9216x14336: 16.9 us against 18.1 at 7 waves; 10240x11008: 14.8 against 15.3 at 11;
@@ -314,7 +322,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   }
   int tiles_per_wg = pair_tiles ? 2 : 1;
   int workgroup_cap = 0;
-  if (!mc && tiles >= kNumCus && ksteps >= 4) {
+  if (!mc && tiles >= cus && ksteps >= 4) {
     // "Exact fit": when the tiles divide (nearly) evenly over the compute units, one workgroup
     // of four waves per compute unit -- one wave per SIMD, all with the same amount of work --
     // beats any over-subscribed launch (8192x8192: 8.7 us against 10.2 us; 28672x8192: 2 %).
@@ -325,12 +333,12 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // 35.5 us with one tile and four waves per workgroup against 38.4 with walks of 7 tiles.)
     const int longest_walk = knobs.wide_waves ? 1 : 7;
     for (int tw = 4; tw >= 1; tw /= 2) {
-      const int sequences = kNumCus * tw;
+      const int sequences = cus * tw;
       if (ceil_div(tiles, sequences) > longest_walk) continue;
       if ((long long)ceil_div(tiles, sequences) * sequences * 100 <= (long long)tiles * 103) {
         tiles_per_wg = tw;
         split_k = 4 / tw;
-        workgroup_cap = kNumCus;
+        workgroup_cap = cus;
         break;
       }
     }
@@ -379,7 +387,7 @@ int check_problem(const void* weights, const void* scale, const void* zero_add, 
   if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
   if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
   if (n_out % 4) return MGEMV_ERR_ROWS;
-  if (k % chunk_k(weight_bits)) return MGEMV_ERR_COLS;
+  if (k % 8) return MGEMV_ERR_COLS;  // utils/preprocess.h:324-327
   if (quant_op == MGEMV_PER_COLUMN_SCALE_ONLY) {
     group_size = k;  // mixed_gemv_test.cu:142-143
   } else {
@@ -421,9 +429,40 @@ hipError_t launch_dequant(const DequantParams& p, int qop, half_t* out, hipStrea
   }
 }
 
+// What the launch path needs to know about a device, looked up once per device and process
+// (the first launch on a device pays for one hipGetDeviceProperties call).
+struct DeviceInfo {
+  bool usable;   // a gfx950 device
+  int num_cus;
+};
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_device_state[kMaxDevices];  // 0 unknown, else 1 + (usable ? num_cus : 0)
+
+// The device a stream belongs to (the null stream: the calling thread's current device).
+int device_of_stream(hipStream_t stream, int& device) {
+  if (stream != nullptr && hipStreamGetDevice(stream, &device) == hipSuccess) return MGEMV_OK;
+  return hipGetDevice(&device) == hipSuccess ? MGEMV_OK : MGEMV_ERR_NO_DEVICE;
+}
+
+int device_info(int device, DeviceInfo& info) {
+  const bool tracked = device >= 0 && device < kMaxDevices;
+  int state = tracked ? g_device_state[device].load(std::memory_order_relaxed) : 0;
+  if (state == 0) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return MGEMV_ERR_NO_DEVICE;
+    const bool usable = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    state = 1 + (usable ? prop.multiProcessorCount : 0);
+    if (tracked) g_device_state[device].store(state, std::memory_order_relaxed);
+  }
+  info.usable = state > 1;
+  info.num_cus = state - 1;
+  return info.usable ? MGEMV_OK : MGEMV_ERR_NO_DEVICE;
+}
+
 // The knobs of a problem with the element type taken into account.
-PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_batch, int act) {
+PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_batch, int act, int num_cus = kNumCus) {
   PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch);
+  knobs.num_cus = num_cus;
   if (act == kActBf16) {
     // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
     // fp32 dequantiser wants the registers of 8-wave workgroups
@@ -438,7 +477,7 @@ PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_ba
 int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
              const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k, int group_size,
              int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
-             int64_t stride_bias, int64_t stride_y, void* stream, int act) {
+             int64_t stride_bias, int64_t stride_y, void* stream, int act, float alpha = 1.0f, float beta = 1.0f) {
   if (batch_count < 1 || batch_count > 65535) return MGEMV_ERR_BATCH;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
@@ -447,19 +486,27 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
       reinterpret_cast<uintptr_t>(bias) % 2)
     return MGEMV_ERR_ALIGNMENT;
   if (stride_weights % 16 || stride_x % 8) return MGEMV_ERR_ALIGNMENT;
+  int device = 0;
+  if (const int st = device_of_stream(static_cast<hipStream_t>(stream), device)) return st;
+  DeviceInfo info{};
+  if (const int st = device_info(device, info)) return st;
 
   GemvLaunch g{};
+  g.device = device;
   g.weights = static_cast<const uint8_t*>(weights);
   g.scale = reinterpret_cast<const half_t*>(scale);
   g.zero_add = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? reinterpret_cast<const half_t*>(zero_add) : nullptr;
   g.n_out = n_out;
   g.k = k;
   g.group_size = group_size;
-  g.plan = plan_launch(n_out, k, weight_bits, m_batch, knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act));
+  g.plan = plan_launch(n_out, k, weight_bits, m_batch,
+                       knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act, info.num_cus));
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
   g.tail.flags = g_dequant_flags.load();
+  g.tail.alpha = alpha;
+  g.tail.beta = beta;
   {
     const int sequences = g.plan.workgroups * g.plan.tiles_per_wg;
     g.tail.seq_base = num_tiles(n_out) / sequences;
@@ -507,6 +554,10 @@ int dequantize_any(const void* weights, const uint16_t* scale, const uint16_t* z
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   if (reinterpret_cast<uintptr_t>(out) % 4) return MGEMV_ERR_ALIGNMENT;
+  int device = 0;
+  if (const int st = device_of_stream(static_cast<hipStream_t>(stream), device)) return st;
+  DeviceInfo info{};
+  if (const int st = device_info(device, info)) return st;
   DequantParams p{};
   p.weights = static_cast<const uint8_t*>(weights);
   p.scale = reinterpret_cast<const half_t*>(scale);
@@ -573,6 +624,82 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
                      int k, int group_size, int quant_op, int weight_bits, void* stream) {
   return mgemv::dequantize_any(weights, scale, zero_add, out, n_out, k, group_size, quant_op, weight_bits, stream,
                                mgemv::kActF16);
+}
+
+// gemv/device/gemv_adaptor.h:114-178 as one plain struct.
+int mgemv_gemv_arguments(const mgemv_arguments* a, void* stream) {
+  if (a == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (a->element != MGEMV_ELEMENT_F16 && a->element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
+  // The operands are the reference's dense ones; a leading dimension may repeat what the reference
+  // passes (mixed_gemv_test.cu:136-140, 153-154) or be 0 = "dense", nothing else.
+  const int64_t n = a->n_out, k = a->k;
+  if (a->lda != 0 && a->lda != 4 * k && a->lda != k) return MGEMV_ERR_LEADING_DIMENSION;
+  if (a->ldb != k && !(a->ldb == 0 && a->m_batch == 1)) return MGEMV_ERR_LEADING_DIMENSION;
+  if (a->ld_scale != 0 && a->ld_scale != n) return MGEMV_ERR_LEADING_DIMENSION;
+  if (a->ld_zero != 0 && a->ld_zero != n) return MGEMV_ERR_LEADING_DIMENSION;
+  if (a->ldc != 0 && a->ldc != n) return MGEMV_ERR_LEADING_DIMENSION;
+  if (a->ldd != 0 && a->ldd != n) return MGEMV_ERR_LEADING_DIMENSION;
+  return mgemv::gemv_any(a->weights, a->x, a->scale, a->zero_add, a->bias, a->y, a->batch_count, a->n_out,
+                         a->m_batch, a->k, a->group_size, a->quant_op, a->weight_bits, a->batch_stride_weights,
+                         a->batch_stride_x, a->batch_stride_scale, a->batch_stride_bias, a->batch_stride_y, stream,
+                         a->element == MGEMV_ELEMENT_BF16 ? mgemv::kActBf16 : mgemv::kActF16, a->alpha, a->beta);
+}
+
+// host/mixed_gemv.h:60-70 on the GPU: un-preprocessed weights and int8 zero points in host
+// memory in, result in host memory out.
+int mgemv_host_gemv(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t* weights,
+                    const uint16_t* x, const uint16_t* scale, const int8_t* zero_point, const uint16_t* bias,
+                    uint16_t* y, int quant_op, int weight_bits) {
+  if (batch != 1) return MGEMV_ERR_BATCH;  // host/mixed_gemv.h:77-80
+  if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
+  if (weights == nullptr || x == nullptr || scale == nullptr || y == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (quant_op != MGEMV_PER_COLUMN_SCALE_ONLY && quant_op != MGEMV_FINEGRAINED_SCALE_ONLY &&
+      quant_op != MGEMV_FINEGRAINED_SCALE_AND_ZEROS)
+    return MGEMV_ERR_QUANT_OP;
+  if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
+  const bool has_zero = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  if (has_zero && zero_point == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
+  if (quant_op == MGEMV_PER_COLUMN_SCALE_ONLY) group_size = k;
+  if (group_size <= 0 || k % group_size) return MGEMV_ERR_GROUP_SIZE;
+  const size_t groups = (size_t)(k / group_size), table = groups * (size_t)n_out;
+
+  const size_t shape[2] = {(size_t)k, (size_t)n_out};
+  const int quant_type = weight_bits == 4 ? MGEMV_W4_A16 : MGEMV_W8_A16;
+  std::vector<uint8_t> tiled(mgemv_preprocessed_size(shape, 2, quant_type));
+  if (const int st = mgemv_preprocess_weights(tiled.data(), weights, shape, 2, MGEMV_COLUMN_MAJOR, quant_type)) return st;
+  std::vector<uint16_t> zero_add;
+  if (has_zero) {
+    zero_add.resize(table);
+    if (const int st = mgemv_fold_zero_points(zero_add.data(), scale, zero_point, table)) return st;  // utils/preprocess.h:94-101
+  }
+
+  // one device allocation, 256-byte aligned pieces
+  auto align = [](size_t v) { return (v + 255) / 256 * 256; };
+  const size_t off_w = 0, off_x = off_w + align(tiled.size()), off_s = off_x + align((size_t)m_batch * k * 2),
+               off_z = off_s + align(table * 2), off_b = off_z + align(has_zero ? table * 2 : 0),
+               off_y = off_b + align(bias ? (size_t)n_out * 2 : 0), total = off_y + align((size_t)m_batch * n_out * 2);
+  uint8_t* dev = nullptr;
+  if (hipMalloc(reinterpret_cast<void**>(&dev), total) != hipSuccess) return MGEMV_ERR_ALLOCATION;
+  int st = MGEMV_OK;
+  auto up = [&](size_t off, const void* src, size_t bytes) {
+    if (st == MGEMV_OK && bytes && hipMemcpy(dev + off, src, bytes, hipMemcpyHostToDevice) != hipSuccess) st = MGEMV_ERR_LAUNCH;
+  };
+  up(off_w, tiled.data(), tiled.size());
+  up(off_x, x, (size_t)m_batch * k * 2);
+  up(off_s, scale, table * 2);
+  if (has_zero) up(off_z, zero_add.data(), table * 2);
+  if (bias) up(off_b, bias, (size_t)n_out * 2);
+  if (st == MGEMV_OK)
+    st = mgemv_gemv(dev + off_w, reinterpret_cast<const uint16_t*>(dev + off_x), reinterpret_cast<const uint16_t*>(dev + off_s),
+                    has_zero ? reinterpret_cast<const uint16_t*>(dev + off_z) : nullptr,
+                    bias ? reinterpret_cast<const uint16_t*>(dev + off_b) : nullptr, reinterpret_cast<uint16_t*>(dev + off_y),
+                    n_out, m_batch, k, group_size, quant_op, weight_bits, nullptr);
+  // the blocking copy on the null stream is ordered behind the kernel
+  if (st == MGEMV_OK && hipMemcpy(y, dev + off_y, (size_t)m_batch * n_out * 2, hipMemcpyDeviceToHost) != hipSuccess)
+    st = MGEMV_ERR_LAUNCH;
+  (void)hipFree(dev);
+  return st;
 }
 
 int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave, int max_workgroups) {
@@ -656,7 +783,16 @@ int mgemv_tuned_plan_clear(void) {
 int mgemv_tuned_plan_count(void) { return mgemv::g_tuned_count.load(); }
 
 namespace {
-int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_size, int act, int out[8]);
+int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_size, int act, int out[8],
+                     int num_cus = mgemv::kNumCus);
+}
+
+int mgemv_query_launch_for(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
+                           int num_compute_units, int out[8]) {
+  if (element != MGEMV_ELEMENT_F16 && element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
+  if (num_compute_units < 1 || num_compute_units > 4096) return MGEMV_ERR_SIZE;
+  return query_launch_any(n_out, m_batch, k, weight_bits, group_size,
+                          element == MGEMV_ELEMENT_BF16 ? mgemv::kActBf16 : mgemv::kActF16, out, num_compute_units);
 }
 
 int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]) {
@@ -668,12 +804,12 @@ int mgemv_query_launch_bf16(int n_out, int m_batch, int k, int weight_bits, int 
 }
 
 namespace {
-int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_size, int act, int out[8]) {
+int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_size, int act, int out[8], int num_cus) {
   if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
   const int st = check_tuned_key(n_out, k, weight_bits, group_size, m_batch);
   if (st != MGEMV_OK) return st;
   const mgemv::LaunchPlan lp = mgemv::plan_launch(
-      n_out, k, weight_bits, m_batch, mgemv::knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act));
+      n_out, k, weight_bits, m_batch, mgemv::knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act, num_cus));
   out[0] = lp.wgs_per_xcd * mgemv::kNumXcd;
   out[1] = lp.threads;
   out[2] = lp.split_k;

@@ -98,8 +98,9 @@ void transpose_quantised(uint8_t* dst, const uint8_t* src, size_t k, size_t n_ou
 }
 
 // Walks the chunks of row n in ascending k and hands each (source byte offset inside the row,
-// byte offset inside the tiled buffer) to `visit`; nested loops instead of chunk_offset() keep
-// integer divisions out of the inner loop.
+// byte offset inside the tiled buffer, bytes of the chunk that lie inside the row -- fewer than 16
+// only for the last chunk of a row whose k is not a multiple of the chunk) to `visit`; nested
+// loops instead of chunk_offset() keep integer divisions out of the inner loop.
 template <typename Visit>
 inline void for_each_chunk_of_row(size_t n, size_t k, size_t ksteps, int bits, Visit visit) {
   const size_t ck = (size_t)mgemv::chunk_k(bits);
@@ -110,7 +111,8 @@ inline void for_each_chunk_of_row(size_t n, size_t k, size_t ksteps, int bits, V
     for (size_t slice = 0; slice < (size_t)mgemv::kKSlices && k0 < k; ++slice) {
       const size_t lane_off = (slice * mgemv::kTileRows + r) * (size_t)mgemv::kChunkBytes;
       for (size_t blk = 0; blk < (size_t)mgemv::kBlocksPerUnit && k0 < k; ++blk, k0 += ck)
-        visit(k0 * (size_t)bits / 8, unit + blk * (size_t)mgemv::kBlockBytes + lane_off);
+        visit(k0 * (size_t)bits / 8, unit + blk * (size_t)mgemv::kBlockBytes + lane_off,
+              (k - k0 < ck ? k - k0 : ck) * (size_t)bits / 8);
     }
   }
 }
@@ -129,9 +131,9 @@ void tile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k, i
 #pragma omp parallel for schedule(static)
   for (long long n = 0; n < (long long)n_out; ++n) {
     const uint8_t* row = src + (size_t)n * row_bytes;
-    for_each_chunk_of_row((size_t)n, k, ksteps, bits, [&](size_t src_off, size_t dst_off) {
-      uint32_t words[4];
-      std::memcpy(words, row + src_off, mgemv::kChunkBytes);
+    for_each_chunk_of_row((size_t)n, k, ksteps, bits, [&](size_t src_off, size_t dst_off, size_t valid) {
+      uint32_t words[4] = {0, 0, 0, 0};  // positions past k: any value, they only ever meet zero activations
+      std::memcpy(words, row + src_off, valid);
       if (bits == 4) {
         for (int j = 0; j < 4; ++j) words[j] = mgemv::encode_int4_word(words[j]);
       } else {
@@ -148,7 +150,7 @@ void untile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k,
 #pragma omp parallel for schedule(static)
   for (long long n = 0; n < (long long)n_out; ++n) {
     uint8_t* row = dst + (size_t)n * row_bytes;
-    for_each_chunk_of_row((size_t)n, k, ksteps, bits, [&](size_t row_off, size_t tiled_off) {
+    for_each_chunk_of_row((size_t)n, k, ksteps, bits, [&](size_t row_off, size_t tiled_off, size_t valid) {
       uint32_t words[4];
       std::memcpy(words, src + tiled_off, mgemv::kChunkBytes);
       if (bits == 4) {
@@ -156,7 +158,7 @@ void untile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k,
       } else {
         for (int j = 0; j < 4; ++j) words[j] = mgemv::decode_int8_word(words[j]);
       }
-      std::memcpy(row + row_off, words, mgemv::kChunkBytes);
+      std::memcpy(row + row_off, words, valid);
     });
   }
 }
@@ -164,7 +166,7 @@ void untile_one_matrix(uint8_t* dst, const uint8_t* src, size_t n_out, size_t k,
 int check_dims(size_t n_out, size_t k, int bits) {
   if (n_out == 0 || k == 0) return MGEMV_ERR_SIZE;
   if (n_out % 4) return MGEMV_ERR_ROWS;                          // utils/preprocess.h:319-322
-  if (k % (size_t)mgemv::chunk_k(bits)) return MGEMV_ERR_COLS;   // one 128-bit access of one row
+  if (k % 8) return MGEMV_ERR_COLS;                              // utils/preprocess.h:324-327
   if (n_out > 0x7fffffffull || k > 0x7fffffffull) return MGEMV_ERR_SIZE;
   return MGEMV_OK;
 }
@@ -176,6 +178,7 @@ extern "C" {
 int mgemv_pack_int4(uint8_t* packed, const int8_t* unpacked, size_t n_unpacked) {
   if (n_unpacked == 0) return MGEMV_OK;
   if (packed == nullptr || unpacked == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (n_unpacked % 2) return MGEMV_ERR_SIZE;  // two elements per byte
   const size_t n_bytes = n_unpacked / 2;
   for (size_t i = 0; i < n_bytes; ++i) {
     const unsigned lo = (unsigned)unpacked[2 * i] & 0xfu;
@@ -282,20 +285,22 @@ const char* mgemv_status_string(int status) {
     case MGEMV_ERR_NULL_POINTER: return "a required pointer is NULL";
     case MGEMV_ERR_RANK: return "weight shape must be 2-D {k, n_out} or 3-D {experts, k, n_out}";
     case MGEMV_ERR_ROWS: return "n_out must be a multiple of 4";
-    case MGEMV_ERR_COLS: return "k must be a multiple of one 128-bit weight access (32 int4 / 16 int8 elements)";
+    case MGEMV_ERR_COLS: return "k must be a multiple of 8";
     case MGEMV_ERR_GROUP_SIZE: return "group_size must be >= 64, a multiple of 32 and divide k";
     case MGEMV_ERR_QUANT_OP: return "quant_op must be 1 (per-column scale), 2 (group scale) or 3 (group scale + zero)";
     case MGEMV_ERR_QUANT_TYPE: return "weights must be int8 (W8_A16) or int4 (W4_A16)";
     case MGEMV_ERR_BATCH: return "batch_count must be >= 1 and m_batch in [1, 16]";
     case MGEMV_ERR_LAYOUT: return "layout must be 0 (row major) or 1 (column major)";
+    case MGEMV_ERR_LEADING_DIMENSION: return "a leading dimension or batch stride describes an operand this library does not take (only the reference's dense operands)";
+    case MGEMV_ERR_ALLOCATION: return "device memory could not be allocated (host-pointer entry point)";
     case MGEMV_ERR_SIZE: return "a dimension is zero, negative or exceeds the 32-bit index range of the kernels";
     case MGEMV_ERR_LAUNCH: return "HIP launch failed";
     case MGEMV_ERR_NO_DEVICE: return "no usable gfx950 device";
-    case MGEMV_ERR_ALIGNMENT: return "device pointer alignment: weights and activations 16 bytes, scales/zeros/bias/output 8 bytes";
+    case MGEMV_ERR_ALIGNMENT: return "device pointer alignment: weights and activations 16 bytes, scales / zeros / bias / outputs 2 bytes, dequantised output 4 bytes";
     default: return "unknown status";
   }
 }
 
-int mgemv_version(void) { return 200; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
+int mgemv_version(void) { return 210; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
 
 }  // extern "C"

@@ -30,6 +30,7 @@ struct GemvTail {
   int m_batch;         // activation rows (matrix-core kernel)
   int num_groups;      // k / group_size (1 in per-column mode): extent of the scale / zero tables
   int flags;           // kExactIntegerFormOnly or 0
+  float alpha, beta;   // epilogue: y = alpha * acc + beta * bias (gemv/device/gemv_adaptor.h:123, epilogue{alpha, beta})
   int seq_base;        // VALU kernel: tiles / sequences ...
   int seq_rem;         // ... and tiles % sequences (the first seq_rem sequences get one tile more)
   long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
@@ -105,6 +106,15 @@ __device__ __forceinline__ bool wave_scales_permit_short_form(const Bits (&scale
   return __builtin_amdgcn_ballot_w64(!ok) == 0;
 }
 
+// Epilogue value before the final rounding: alpha * acc + beta * bias in fp32, the outer
+// multiply-add fused -- what the reference's LinearCombination computes (alpha * accumulator +
+// source, epilogue/threadblock/epilogue.h:64, 93; one `a * b + c` per element, which nvcc
+// contracts).  With alpha = beta = 1 this is the single rounded fp32 add of
+// host/mixed_gemv.h:102-103, bit for bit, and without a bias it adds +0 as the reference does.
+__device__ __forceinline__ float epilogue_value(const GemvTail& tail, float acc, bool has_bias, float bias) {
+  return __builtin_fmaf(tail.alpha, acc, has_bias ? tail.beta * bias : 0.0f);
+}
+
 // Sum over the four k slices of a wave: lanes l, l+16, l+32, l+48 hold the same row.
 // The result is valid in lanes 0..15.
 __device__ __forceinline__ float reduce_k_slices(float v) {
@@ -153,6 +163,7 @@ struct GemvLaunch {
   dim3 grid, block;
   size_t lds;
   hipStream_t stream;
+  int device;  // the device `stream` belongs to
 };
 
 // Dispatchers, one translation unit each (the kernels are templates on weight width, quant mode,

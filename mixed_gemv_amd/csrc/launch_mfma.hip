@@ -46,11 +46,13 @@ __device__ __forceinline__ void load_activations_mfma(MfmaActivations<BITS>& f, 
 #pragma unroll
   for (int i = 0; i < kBlocksPerUnit; ++i) {
     const int k_block = k_run + i * G::kChunkK;
-    // Batch rows past m_batch and reduction positions past k fall outside the descriptor and
-    // read as zero (k is a multiple of the chunk, so a block is wholly inside or outside).
-    const uint32_t off = k_block < p.k ? (uint32_t)(m * p.k + k_block) * 2u : 0xfffffff0u;
+    // Batch rows past m_batch fall outside the descriptor and read as zero; reduction positions
+    // past k are sent there (k is a multiple of 8, so each 128-bit piece is wholly inside or outside).
 #pragma unroll
-    for (int j = 0; j < kFrags; ++j) f.x[i][j] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, j * 16, kCacheDefault);
+    for (int j = 0; j < kFrags; ++j) {
+      const uint32_t off = k_block + j * 8 < p.k ? (uint32_t)(m * p.k + k_block + j * 8) * 2u : 0xfffffff0u;
+      f.x[i][j] = __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, kCacheDefault);
+    }
   }
 }
 
@@ -301,8 +303,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
         for (int v = 0; v < 4; ++v) {
           const int n = n0 + v;
           if (n < p.n_out) {
-            float r = sum[v];
-            if (has_bias) r += (float)tail.bias[n];
+            const float r = epilogue_value(tail, sum[v], has_bias, has_bias ? (float)tail.bias[n] : 0.0f);
             tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
           }
         }
@@ -320,8 +321,7 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
       for (int v = 0; v < 4; ++v) {
         const int n = n0 + v;
         if (n < p.n_out) {
-          float r = acc[t][v];
-          if (has_bias) r += (float)tail.bias[n];
+          const float r = epilogue_value(tail, acc[t][v], has_bias, has_bias ? (float)tail.bias[n] : 0.0f);
           tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
         }
       }
@@ -556,12 +556,12 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
     for (int v = 0; v < 4; ++v) {
       const int n = n0 + v;
       if (n < p.n_out) {
-        float r = sum[v];
         if constexpr (ACT == kActBf16) {
-          if (has_bias) r += bf16_low_to_f32(reinterpret_cast<const uint16_t*>(tail.bias)[n]);
+          const float b = has_bias ? bf16_low_to_f32(reinterpret_cast<const uint16_t*>(tail.bias)[n]) : 0.0f;
+          const float r = epilogue_value(tail, sum[v], has_bias, b);
           reinterpret_cast<uint16_t*>(tail.y)[(size_t)m * (size_t)p.n_out + n] = (uint16_t)pack_bf16(r, 0.0f);
         } else {
-          if (has_bias) r += (float)tail.bias[n];
+          const float r = epilogue_value(tail, sum[v], has_bias, has_bias ? (float)tail.bias[n] : 0.0f);
           tail.y[(size_t)m * (size_t)p.n_out + n] = (half_t)r;
         }
       }
@@ -623,8 +623,7 @@ hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
     constexpr int kMaxDevices = 64;
     static std::atomic<int> granted[kMaxDevices];
     static std::mutex grant_mutex;
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess) return hipErrorInvalidDevice;
+    const int device = g.device;  // the device of the launch stream, not the calling thread's current one
     const bool tracked = device >= 0 && device < kMaxDevices;
     if (!tracked || granted[device].load() < (int)g.lds) {
       std::lock_guard<std::mutex> lock(grant_mutex);  // grant and bookkeeping change together

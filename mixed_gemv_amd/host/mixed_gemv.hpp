@@ -114,9 +114,20 @@ struct TensorRef {
   int stride() const { return ld; }
 };
 
+// cutlass::epilogue::thread::LinearCombination<...>::Params as the reference's Arguments carry it
+// (gemv/device/gemv_adaptor.h:123; mixed_gemv_test.cu:72-81): D = alpha * accumulator + beta * C.
+// The reference's `{}` is alpha = 1, beta = 0 with a scaling type that never reads C; here beta
+// only matters when ref_C is set, and defaults to 1 so that ref_C is the bias of
+// host/mixed_gemv.h:102-103.
+struct EpilogueParams {
+  float alpha = 1.0f;
+  float beta = 1.0f;
+};
+
 // gemv/device/gemv_adaptor.h:114-261.  Reference letters: M = output features, N = activation
-// rows, K = reduction.  The leading dimensions are accepted for source compatibility; the
-// kernels use dense operands (scale/zero/C/D with ld = M, activations with row stride K).
+// rows, K = reduction.  The operands are dense: a leading dimension must be 0 or the value the
+// reference's caller passes (ref_A 4K, ref_B 0 for one row or K, the others M); any other value
+// is refused with MGEMV_ERR_LEADING_DIMENSION instead of being ignored.
 class GemvAdaptor {
  public:
   struct Arguments {
@@ -127,6 +138,7 @@ class GemvAdaptor {
     TensorRef<const half_t> ref_zero_point;  // folded -z*s
     TensorRef<const half_t> ref_C;           // optional bias, nullptr = none
     TensorRef<half_t> ref_D;
+    EpilogueParams epilogue;
     int group_size = 64;
     int batch_count = 1;
     long long batch_stride_A = 0;            // BYTES of the preprocessed buffer
@@ -147,13 +159,35 @@ class GemvAdaptor {
   void run(void* stream = nullptr) {
     if (!initialized_) throw std::logic_error("GemvAdaptor::run before initialize");
     const Arguments& a = args_;
-    const half_t* zero = hasZero(quant_op_) ? a.ref_zero_point.ptr : nullptr;  // mixed_gemv_test.cu:145-147
-    const auto gemv = element_ == ElementType::kBFloat16 ? mgemv_gemv_batched_bf16 : mgemv_gemv_batched;
-    check(gemv(a.ref_A.ptr, a.ref_B.ptr, a.ref_scale.ptr, zero, a.ref_C.ptr, a.ref_D.ptr, a.batch_count,
-               a.problem_size.m(), a.problem_size.n(), a.problem_size.k(), a.group_size,
-               static_cast<int>(quant_op_), weight_bits_, a.batch_stride_A, a.batch_stride_B,
-               a.batch_stride_scale, a.batch_stride_C, a.batch_stride_D, stream),
-          "GemvAdaptor::run");
+    mgemv_arguments c{};
+    c.n_out = a.problem_size.m();
+    c.m_batch = a.problem_size.n();
+    c.k = a.problem_size.k();
+    c.weights = a.ref_A.ptr;
+    c.lda = a.ref_A.ld;
+    c.x = a.ref_B.ptr;
+    c.ldb = a.ref_B.ld == 0 && c.m_batch > 1 ? c.k : a.ref_B.ld;  // the reference's stride-0 single row, repeated per row
+    c.scale = a.ref_scale.ptr;
+    c.ld_scale = a.ref_scale.ld;
+    c.zero_add = hasZero(quant_op_) ? a.ref_zero_point.ptr : nullptr;  // mixed_gemv_test.cu:145-147
+    c.ld_zero = a.ref_zero_point.ld;
+    c.bias = a.ref_C.ptr;
+    c.ldc = a.ref_C.ld;
+    c.y = a.ref_D.ptr;
+    c.ldd = a.ref_D.ld;
+    c.alpha = a.epilogue.alpha;
+    c.beta = a.epilogue.beta;
+    c.group_size = a.group_size;
+    c.batch_count = a.batch_count;
+    c.batch_stride_weights = a.batch_stride_A;
+    c.batch_stride_x = a.batch_stride_B;
+    c.batch_stride_scale = a.batch_stride_scale;
+    c.batch_stride_bias = a.batch_stride_C;
+    c.batch_stride_y = a.batch_stride_D;
+    c.quant_op = static_cast<int>(quant_op_);
+    c.weight_bits = weight_bits_;
+    c.element = element_ == ElementType::kBFloat16 ? MGEMV_ELEMENT_BF16 : MGEMV_ELEMENT_F16;
+    check(mgemv_gemv_arguments(&c, stream), "GemvAdaptor::run");
   }
 
   void operator()(const Arguments& args, void* stream = nullptr) {
@@ -190,6 +224,43 @@ inline void device_gemv(const void* ptr_A, const half_t* ptr_B, const half_t* pt
   GemvAdaptor op(quant_op, weight_bits, element);
   op.initialize(args);
   op.run(stream);
+}
+
+namespace host {
+namespace reference {
+
+// host::reference::MixedGemv (host/mixed_gemv.h:23-105) with the GPU behind it: operator() has
+// the reference's argument list and meaning -- UN-preprocessed packed weights [M][K], int8 zero
+// points, optional bias, host pointers -- and runs preprocess, zero fold, upload, the device GEMV
+// and the download.  The reference's template parameters that select the instantiation (int4
+// weights with zero points is the only one it defines) are constructor arguments.
+class MixedGemv {
+ public:
+  explicit MixedGemv(WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4)
+      : quant_op_(quant_op), weight_bits_(weight_bits) {}
+
+  // A: packed weights as vector_subbyte<int4b_t>::data() holds them (utils/vector_subbyte.h:150-156), or int8.
+  void operator()(int32_t batch, int32_t M, int32_t N, int32_t K, int32_t group_size, const uint8_t* A, const half_t* B,
+                  const half_t* scale, const int8_t* zero_point, const half_t* bias, half_t* output) const {
+    check(mgemv_host_gemv(batch, M, N, K, group_size, A, B, scale, zero_point, bias, output,
+                          static_cast<int>(quant_op_), weight_bits_),
+          "host::reference::MixedGemv");
+  }
+
+ private:
+  WeightOnlyQuantOp quant_op_;
+  int weight_bits_;
+};
+
+}  // namespace reference
+}  // namespace host
+
+// mixed_gemv_test.cu:167-181: the HOST_CHECK call site.
+inline void host_gemv(const uint8_t* ptr_A, const half_t* ptr_B, const half_t* ptr_scale, const int8_t* ptr_zero_point,
+                      const half_t* ptr_C, half_t* ptr_D, int B, int M, int N, int K, int group_size,
+                      WeightOnlyQuantOp quant_op = WeightOnlyQuantOp::FINEGRAINED_SCALE_AND_ZEROS, int weight_bits = 4) {
+  host::reference::MixedGemv op(quant_op, weight_bits);
+  op(B, M, N, K, group_size, ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D);
 }
 
 }  // namespace mixed_gemv

@@ -1,0 +1,114 @@
+"""The rest of the drop-in boundary on the GPU, all through the C-ABI: the HOST_CHECK-shaped entry
+(host/mixed_gemv.h:60-70), the Arguments-struct entry with the epilogue's alpha / beta
+(gemv/device/gemv_adaptor.h:114-178), reductions that are a multiple of 8 but not of a 128-bit
+chunk (utils/preprocess.h:324-327), and weights preprocessed from row-major input
+(utils/preprocess.h:507-511)."""
+import numpy as np
+import pytest
+
+import mixed_gemv_amd as mg
+import oracle as orc
+from helpers import PER_COLUMN, SCALE_AND_ZEROS, SCALE_ONLY, DeviceProblem, Problem, error_report
+
+pytestmark = pytest.mark.gpu
+REL_TOL = 2e-3  # fp16 outputs within max relative error 2e-3 of the CPU oracle (denominator floor: helpers.error_report)
+
+
+@pytest.mark.parametrize("tag,n_out,k,bits,qop,g,m_batch,bias", [
+    ("h_i4_sz", 512, 2048, 4, SCALE_AND_ZEROS, 128, 1, True),     # the one instantiation the reference defines (host/mixed_gemv.h:23-42)
+    ("h_i4_sz_nobias", 100, 1120, 4, SCALE_AND_ZEROS, 160, 1, False),
+    ("h_i4_sz_rows", 256, 1024, 4, SCALE_AND_ZEROS, 64, 3, True),
+    ("h_i4_s", 128, 1024, 4, SCALE_ONLY, 128, 1, True),
+    ("h_i8_col", 256, 1024, 8, PER_COLUMN, 0, 1, True),
+])
+def test_host_gemv_is_the_host_check_call_site_on_the_gpu(gpu, tag, n_out, k, bits, qop, g, m_batch, bias):
+    """Un-preprocessed weights and int8 zero points in, result out: against the oracle's literal
+    int8-zero path (host/mixed_gemv.h:92-96 as written)."""
+    prob = Problem(tag, n_out, k, bits, qop, g, m_batch=m_batch, bias=bias, scale_range=(0.1, 0.3), zero_kind="int8")
+    y = mg.host_gemv(prob.w_raw, prob.x, prob.scale, prob.zeros_i8, prob.bias, 1, n_out, m_batch, k, prob.group_size,
+                     qop, bits)
+    ref = prob.oracle_gemv(threads=8, literal_int8_zero=True)
+    _, rel, _ = error_report(y, ref)
+    assert rel <= REL_TOL
+    # the same numbers as the device entry fed by hand
+    dev = DeviceProblem(prob, gpu)
+    assert np.array_equal(dev.run().view(np.uint16), y.view(np.uint16))
+
+
+def _run_arguments(dev, prob, alpha=1.0, beta=1.0, leading_dims=None):
+    import torch
+    dev.y.fill_(0x7e00)
+    mg.gemv_arguments(dev.w, dev.x, dev.scale, dev.zero, dev.bias, dev.y, prob.n_out, prob.m_batch, prob.k,
+                      prob.group_size, prob.quant_op, prob.bits, alpha=alpha, beta=beta, leading_dims=leading_dims,
+                      element=prob.element)
+    torch.cuda.synchronize()
+    return dev.y.cpu().numpy().view(np.float16)
+
+
+@pytest.mark.parametrize("m_batch", [1, 3, 8])   # VALU kernel, VALU with several rows, matrix cores
+def test_arguments_entry_alpha_beta(gpu, m_batch):
+    prob = Problem("a_ab", 256, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=m_batch, bias=True, x_dist="normal")
+    dev = DeviceProblem(prob, gpu)
+    plain = dev.run().copy()
+    # alpha = beta = 1 with the reference's own leading dimensions (mixed_gemv_test.cu:136-140) is the plain entry, bit for bit
+    lds = (4 * prob.k, prob.k if m_batch > 1 else 0, prob.n_out, prob.n_out, prob.n_out, prob.n_out)
+    assert np.array_equal(_run_arguments(dev, prob, leading_dims=lds).view(np.uint16), plain.view(np.uint16))
+    # beta = 0 drops the bias: equals the launch without one
+    nobias = DeviceProblem(Problem("a_ab", 256, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=m_batch, bias=False,
+                                   x_dist="normal"), gpu)
+    acc16 = nobias.run().copy()
+    assert np.array_equal(_run_arguments(dev, prob, beta=0.0).view(np.uint16), acc16.view(np.uint16))
+    # a power of two commutes with the final rounding (no result here is subnormal after halving)
+    half = _run_arguments(dev, prob, alpha=0.5, beta=0.0)
+    big = np.abs(acc16.astype(np.float32)) >= 2.0 ** -13
+    assert np.array_equal(half[big].view(np.uint16), (acc16[big].astype(np.float32) * 0.5).astype(np.float16).view(np.uint16))
+    # general alpha, beta: alpha * acc + beta * bias with one rounding; acc16 is acc rounded to fp16, so allow its half ulp
+    got = _run_arguments(dev, prob, alpha=-1.75, beta=3.0).astype(np.float64)
+    want = -1.75 * acc16.astype(np.float64) + 3.0 * prob.bias.astype(np.float64)[None, :]
+    tol = 2.0 ** -10 * (1.75 * np.abs(acc16.astype(np.float64)) + np.abs(want)) + 2.0 ** -24
+    assert np.all(np.abs(got - want) <= tol)
+
+
+def test_arguments_entry_bias_term_alone_is_exact(gpu):
+    """x = 0: y = fp16(beta * bias) exactly (epilogue/threadblock/epilogue.h:64)."""
+    import torch
+    prob = Problem("a_bias", 128, 1024, 4, SCALE_AND_ZEROS, 128, bias=True)
+    dev = DeviceProblem(prob, gpu)
+    dev.x = torch.zeros_like(dev.x)
+    for alpha, beta in ((1.0, 1.0), (5.0, 0.37), (0.0, -2.0)):
+        y = _run_arguments(dev, prob, alpha=alpha, beta=beta)[0]
+        want = (np.float32(beta) * prob.bias.astype(np.float32)).astype(np.float16)
+        assert np.array_equal(y.view(np.uint16), want.view(np.uint16)), (alpha, beta)
+
+
+@pytest.mark.parametrize("bits,k", [(4, 4104), (4, 520), (4, 8), (8, 1048), (8, 264)])
+@pytest.mark.parametrize("m_batch", [1, 4, 8])
+def test_reduction_length_a_multiple_of_8_only(gpu, bits, k, m_batch):
+    """Per-column mode with k % 8 == 0 but not a whole 128-bit chunk per row: the preprocessor pads
+    the last chunk, the kernels never multiply the padding by a non-zero activation."""
+    prob = Problem(f"k8_{bits}_{k}", 96, k, bits, PER_COLUMN, 0, m_batch=m_batch, bias=True, x_dist="normal")
+    dev = DeviceProblem(prob, gpu)
+    assert np.array_equal(dev.dequant().view(np.uint16), prob.oracle_dequant().view(np.uint16))
+    y = dev.run()
+    _, rel, _ = error_report(y, prob.oracle_gemv(threads=8))
+    assert rel <= REL_TOL
+
+
+@pytest.mark.parametrize("bits,qop,g", [(4, SCALE_AND_ZEROS, 128), (8, PER_COLUMN, 0)])
+def test_weights_preprocessed_from_row_major_input(gpu, bits, qop, g):
+    """utils/preprocess.h:507-511: a [k][n_out] row-major matrix is transposed first.  The buffer the
+    kernels consume must be the one the column-major route produces, and the GEMV over it must pass."""
+    import torch
+    n_out, k = 320, 1536
+    prob = Problem(f"rm_{bits}", n_out, k, bits, qop, g, bias=True)
+    q = prob.q.reshape(n_out, k)
+    qt = mg.QuantType.W4_A16 if bits == 4 else mg.QuantType.W8_A16
+    q_rm = np.ascontiguousarray(q.T)                                   # [k][n_out]
+    raw_rm = orc.pack_int4(q_rm.reshape(-1)) if bits == 4 else q_rm.view(np.uint8).reshape(-1)
+    pre = mg.MixedGemvWeightPreprocessor.run(raw_rm, (k, n_out), mg.LayoutType.kRowMajor, qt)
+    dev = DeviceProblem(prob, gpu)
+    assert np.array_equal(pre, dev.w.cpu().numpy())
+    dev.w = torch.from_numpy(pre).to(gpu)
+    assert np.array_equal(dev.dequant().view(np.uint16), prob.oracle_dequant().view(np.uint16))
+    _, rel, _ = error_report(dev.run(), prob.oracle_gemv(threads=8))
+    assert rel <= REL_TOL

@@ -29,8 +29,8 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(handle, name), f"{name} declared in include/mixed_gemv.h but not exported"
     assert declared == set(_lib.SIGNATURES), "python binding and header disagree"
     assert _lib.lib().mgemv_version() >= 100
-    for code in range(0, 14):
-        assert _lib.lib().mgemv_status_string(code)
+    for code in range(0, 16):
+        assert _lib.lib().mgemv_status_string(code) not in (None, b"", b"unknown status")
 
 
 def test_pack_unpack_and_fold_equal_the_oracle():
@@ -153,8 +153,8 @@ def test_preprocess_error_codes():
         ((64,), COL, W4, 2),            # rank 1          utils/preprocess.h:486-489
         ((1, 2, 64, 64), COL, W4, 2),   # rank 4
         ((64, 6), COL, W4, 3),          # rows % 4        utils/preprocess.h:319-322
-        ((40, 64), COL, W4, 4),         # k % 32 (int4)   utils/preprocess.h:324-327
-        ((24, 64), COL, W8, 4),         # k % 16 (int8)
+        ((36, 64), COL, W4, 4),         # k % 8           utils/preprocess.h:324-327
+        ((20, 64), COL, W8, 4),
         ((64, 64), COL, mg.QuantType.W4_AFP8, 7),
         ((64, 64), 5, W4, 9),
         ((0, 64), COL, W4, 10),
@@ -169,6 +169,8 @@ def test_preprocess_error_codes():
     assert lib.mgemv_preprocess_weights(None, None, shape, 2, 1, 1) == 1
     assert lib.mgemv_pack_int4(None, None, 8) == 1
     assert lib.mgemv_pack_int4(None, None, 0) == 0
+    three = np.zeros(3, dtype=np.int8)
+    assert lib.mgemv_pack_int4(ctypes.c_void_p(buf.ctypes.data), ctypes.c_void_p(three.ctypes.data), 3) == 10  # odd count
     assert lib.mgemv_fold_zero_points(None, None, None, 4) == 1
 
 
@@ -186,7 +188,8 @@ def test_gemv_argument_checks_return_codes_without_launching():
     assert gemv(m=0) == 8 and gemv(m=17) == 8              # the reference accepts N == 1 only (host/mixed_gemv.h:72-75)
     assert gemv(n_out=0) == 10 and gemv(k=-4) == 10
     assert gemv(n_out=66) == 3
-    assert gemv(k=520) == 4
+    assert gemv(k=516) == 4                                 # k % 8 (utils/preprocess.h:324-327)
+    assert gemv(k=520, qop=1) != 4                          # a multiple of 8 passes the shape checks (per-column mode)
     assert gemv(g=32) == 5                                  # gemv/device/gemv_adaptor.h:199-203
     assert gemv(g=96, k=512) == 5                           # does not divide k
     assert gemv(g=80, k=640) == 5                           # not a multiple of 32
@@ -208,6 +211,78 @@ def test_gemv_argument_checks_return_codes_without_launching():
     assert lib.mgemv_set_matrix_core_threshold(18) == 8
     assert lib.mgemv_set_matrix_core_variant(3) == 10 and lib.mgemv_set_matrix_core_variant(0) == 0
     assert lib.mgemv_set_dequant_form(2) == 10 and lib.mgemv_set_dequant_form(0) == 0
+
+
+@pytest.mark.parametrize("bits,n_out,k", [(4, 20, 40), (4, 64, 8), (4, 36, 1000), (8, 12, 24), (8, 32, 520)])
+def test_k_that_is_a_multiple_of_8_only_round_trips(bits, n_out, k):
+    """utils/preprocess.h:324-327 asks for k % 8 == 0, not for whole 128-bit chunks: the last chunk
+    of a row may be partly padding."""
+    qt = W4 if bits == 4 else W8
+    raw = orc.fill_int8(n_out * k * bits // 8, 11, -128, 127).view(np.uint8)
+    pre = mg.MixedGemvWeightPreprocessor.run(raw, (k, n_out), COL, qt)
+    assert pre.size == mg.preprocessed_size((k, n_out), qt)
+    assert np.array_equal(mg.unpreprocess_weights(pre, (k, n_out), qt), raw)
+    # row-major input of the same matrix gives the same buffer
+    q = mg.SubBytePacker.unpack(raw) if bits == 4 else raw.view(np.int8)
+    qt_rm = np.ascontiguousarray(q.reshape(n_out, k).T)
+    raw_rm = mg.SubBytePacker.pack(qt_rm.reshape(-1)) if bits == 4 else qt_rm.view(np.uint8).reshape(-1)
+    assert np.array_equal(mg.MixedGemvWeightPreprocessor.run(raw_rm, (k, n_out), ROW, qt), pre)
+
+
+def test_arguments_entry_refuses_operands_that_are_not_dense():
+    """GemvAdaptor::Arguments carries leading dimensions (gemv/device/gemv_adaptor.h:116-122); only the
+    dense values are taken, everything else is a status, before anything touches a GPU."""
+    from mixed_gemv_amd.api import _Arguments
+    lib = _lib.lib()
+    n, m, k = 64, 1, 512
+
+    def call(**over):
+        f = dict(n_out=n, m_batch=m, k=k, weights=0x1000, lda=4 * k, x=0x1000, ldb=0, scale=0x1000, ld_scale=n,
+                 zero_add=0x1000, ld_zero=n, bias=0, ldc=n, y=0x1000, ldd=n, alpha=1.0, beta=1.0, group_size=128,
+                 batch_count=1, batch_stride_weights=0, batch_stride_x=0, batch_stride_scale=0, batch_stride_bias=0,
+                 batch_stride_y=0, quant_op=3, weight_bits=4, element=0)
+        f.update(over)
+        a = _Arguments(**f)
+        return lib.mgemv_gemv_arguments(ctypes.byref(a), None)
+
+    assert lib.mgemv_gemv_arguments(None, None) == 1
+    for field, bad in (("lda", 2 * k), ("ldb", k + 8), ("ld_scale", n + 4), ("ld_zero", 2 * n), ("ldc", 1), ("ldd", n + 64)):
+        assert call(**{field: bad}) == 14, field
+    assert call(m_batch=2, ldb=0) == 14          # stride-0 activations are the reference's single row only
+    assert call(element=2) == 7
+    # dense operands pass the leading-dimension checks and fail later, on the missing device or not at all
+    assert call() in (0, 12)
+    assert call(lda=0, ldb=k, ld_scale=0, ld_zero=0, ldc=0, ldd=0) in (0, 12)
+    assert call(k=516, lda=0) == 4 and call(group_size=32) == 5      # the checks of mgemv_gemv still apply
+
+
+def test_device_entry_points_report_a_missing_device():
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lib = _lib.lib()
+    p = ctypes.c_void_p(0x1000)
+    assert lib.mgemv_gemv(p, p, p, p, None, p, 64, 1, 512, 128, 3, 4, None) == 12
+    assert lib.mgemv_dequantize(p, p, p, p, 64, 512, 128, 3, 4, None) == 12
+
+
+def test_host_gemv_checks_its_arguments_before_touching_the_device():
+    lib = _lib.lib()
+    w = np.zeros(64 * 512 // 2, dtype=np.uint8)
+    h = np.zeros(64 * 512, dtype=np.uint16)
+    z = np.zeros(64 * 4, dtype=np.int8)
+    ptr = lambda a: ctypes.c_void_p(a.ctypes.data)  # noqa: E731
+
+    def call(batch=1, n=64, m=1, k=512, g=128, ww=w, x=h, s=h, zz=z, y=h, qop=3, bits=4):
+        return lib.mgemv_host_gemv(batch, n, m, k, g, ptr(ww) if ww is not None else None, ptr(x), ptr(s),
+                                   ptr(zz) if zz is not None else None, None, ptr(y), qop, bits)
+
+    assert call(batch=2) == 8                      # host/mixed_gemv.h:77-80
+    assert call(m=0) == 8 and call(m=17) == 8      # host/mixed_gemv.h:72-75 takes N == 1 only; here up to 16 rows
+    assert call(ww=None) == 1 and call(zz=None) == 1
+    assert call(qop=0) == 6 and call(bits=3) == 7
+    assert call(g=100) == 5
+    assert call(n=66) == 3 and call(k=516, g=516) == 4
 
 
 def test_tuned_plan_table_steers_exactly_its_problem(tmp_path):
