@@ -9,7 +9,9 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_DIR = os.path.join(PKG_DIR, "lib")
+OBJ_DIR = os.path.join(LIB_DIR, "obj")   # objects and the compiler's intermediate files (the device assembly among them)
 LIB_PATH = os.path.join(LIB_DIR, "libmixed_gemv_amd.so")
+LINT_REPORT = os.path.join(LIB_DIR, "isa_lint.json")
 
 # One translation unit per family of kernel instantiations, so that they compile side by side.
 SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "gemv_kernels.hip", "host_utils.cpp"]
@@ -34,13 +36,32 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
-def build_library(verbose=True, extra_flags=(), jobs=None):
-    os.makedirs(LIB_DIR, exist_ok=True)
+def lint_device_code(verbose=True):
+    """Runs isa_lint over the device assembly the compiler left beside the objects and writes the
+    report next to the library; raises if the compiled code has a hazard the compiler cannot see."""
+    import glob
+    import json
+    from . import isa_lint
+    files = sorted(glob.glob(os.path.join(OBJ_DIR, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+    reports = [isa_lint.lint_file(f) for f in files]
+    with open(LINT_REPORT, "w") as f:
+        json.dump(reports, f, indent=1)
+    bad = sum(len(r["findings"]) for r in reports)
+    if verbose:
+        print(f"isa_lint: {sum(r['dot_instructions'] for r in reports)} dot instructions in "
+              f"{sum(r['kernels_with_dots'] for r in reports)} kernels of {len(files)} files, {bad} findings", flush=True)
+    if bad:
+        raise RuntimeError(f"isa_lint: {bad} hazards in the compiled kernels, see {LINT_REPORT}")
+    return reports
+
+
+def build_library(verbose=True, extra_flags=(), jobs=None, lint=True):
+    os.makedirs(OBJ_DIR, exist_ok=True)
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
 
     def compile_one(src):
-        obj = os.path.join(LIB_DIR, os.path.splitext(src)[0] + ".o")
-        cmd = [hipcc(), *HIP_FLAGS, *extra_flags, "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC,
+        obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+        cmd = [hipcc(), *HIP_FLAGS, *extra_flags, "-save-temps=obj", "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC,
                "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -53,6 +74,8 @@ def build_library(verbose=True, extra_flags=(), jobs=None):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
+    if lint:
+        lint_device_code(verbose)
     return LIB_PATH
 
 

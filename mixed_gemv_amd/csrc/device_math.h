@@ -157,7 +157,12 @@ __device__ __forceinline__ half2_t dequant_pair(half2_t q, half2_t s, half2_t z)
 // (gemv/threadblock/dq_mma_base.h:76-103).
 //
 // The x operand must come straight from a memory load: a VALU write followed within two
-// instructions by a DPP read of the same register is a hazard the assembler does not pad.
+// instructions by a DPP read of the same register is a hazard that neither the assembler nor
+// the compiler (which sees an opaque asm statement) pads.  Nothing in the sources can stop the
+// register allocator from copying x or the accumulator at a bad place, so the build checks the
+// compiled code instead: isa_lint.py walks the device assembly of every kernel and fails the
+// build on a VALU write within two wait states in front of a DPP read, or a read of a dot
+// result by any other kind of instruction within three behind it.
 template <int SRC>
 __device__ __forceinline__ void dot2_row_bcast(float& acc, uint32_t x, half2_t d) {
   static_assert(SRC >= 0 && SRC < 16, "source lane within a 16-lane DPP row");
