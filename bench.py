@@ -293,30 +293,98 @@ def time_workload(wl, steps, warmup, use_graph=False, repetitions=None):
     return statistics.median(walls), statistics.median(events), steps, done, reps, min(walls)
 
 
-def launch_floor_us(device):
-    """Cadence of the smallest possible kernel (a one-element fill) replayed from a HIP graph like the
-    timed steps: what one launch costs on this machine before it reads a single byte."""
+class _Launches:
+    """Anything with launch(i) and rotation(): lets time_workload time a probe like a workload."""
+
+    def __init__(self, fn, rotation):
+        self.fn, self.rot = fn, rotation
+
+    def launch(self, i):
+        self.fn(i)
+
+    def rotation(self):
+        return self.rot
+
+
+def launch_floor_us(use_graph=True):
+    """Cadence of an EMPTY kernel launched like the timed steps: what one launch costs on this
+    machine before it reads a single byte."""
+    import mixed_gemv_amd as mg
+    probe = _Launches(lambda i: mg.probe_empty_launch(), 1)
+    _, ev_us, *_ = time_workload(probe, 2000, 100, use_graph=use_graph, repetitions=7)
+    return ev_us
+
+
+def ceilings_of(wl, use_graph, timeline=False):
+    """What bounds the workload's kernel from above, measured with the probes of the library on
+    the workload's own (rotated, cold) buffers:
+      stream_read   a plain streaming read of exactly the workload's weight bytes, for the launch
+                    shape of the GEMV and for the best of a few others (no scales, no activations,
+                    no arithmetic): us per launch and GB/s of the bytes read;
+      loads_only    the GEMV kernel itself with every load kept and the arithmetic removed;
+      timeline      (headline only) when the phases of one launch happen."""
+    import statistics
     import torch
-    cell = torch.zeros(1, dtype=torch.int32, device=device)
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    graph = torch.cuda.CUDAGraph()
-    with torch.cuda.stream(side):
-        with torch.cuda.graph(graph, stream=side):
-            for _ in range(64):
-                cell.fill_(1)
-    torch.cuda.current_stream().wait_stream(side)
-    for _ in range(20):
-        graph.replay()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(100):
-        graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / 6400
+    import mixed_gemv_amd as mg
+    if wl.bits != 4 or wl.quant_op != 3 or wl.m_batch != 1:
+        return None
+    plan = mg.query_launch(wl.n_out, 1, wl.k, 4, wl.group)
+    w_bytes = wl.w[0].numel()
+    sink = torch.zeros(1, dtype=torch.int32, device=wl.y.device)
+    out = {"weight_bytes": w_bytes, "algorithmic_bytes": wl.bytes, "stream_read": []}
+    waves = plan["threads"] // 64
+    shapes = [("the GEMV's launch shape", plan["workgroups"], waves, 2)]
+    shapes += [("", 128, 8, 2), ("", 256, 8, 2), ("", 512, 4, 4), ("", 1024, 4, 4), ("", 512, 8, 8)]
+    for label, wgs, wv, depth in shapes:
+        if w_bytes // 4096 < wgs * wv * depth:
+            continue
+        probe = _Launches(lambda i, a=(wgs, wv, depth): mg.probe_stream_read(wl.w[i % wl.sets], w_bytes, *a, sink), wl.sets)
+        _, ev_us, *_ = time_workload(probe, 400, 20, use_graph=use_graph, repetitions=5)
+        read = (w_bytes // 4096 // (wgs * wv)) * (wgs * wv) * 4096
+        out["stream_read"].append({"workgroups": wgs, "waves_per_workgroup": wv, "units_in_flight": depth,
+                                   "us_per_launch": round(ev_us, 3), "GBps": round(read / ev_us / 1e3, 1),
+                                   "frac_of_hbm_peak": round(read / ev_us / 1e3 / HBM_PEAK_GBS, 4), "note": label})
+    best = min(out["stream_read"], key=lambda e: e["us_per_launch"])
+    out["stream_read_best_us"] = best["us_per_launch"]
+    # the whole workload at the best plain-read rate: the time below which no kernel of this kind gets
+    out["algorithmic_bytes_at_best_stream_rate_us"] = round(wl.bytes / (best["GBps"] * 1e3), 3)
+    probe = _Launches(lambda i: mg.probe_gemv(mg.PROBE_LOADS_ONLY, None, wl.w[i % wl.sets], wl.x, wl.s[i % wl.sets],
+                                              wl.z[i % wl.sets], wl.y, wl.n_out, wl.k, wl.group), wl.sets)
+    _, ev_us, *_ = time_workload(probe, 400, 20, use_graph=use_graph, repetitions=5)
+    out["loads_only"] = {"us_per_launch": round(ev_us, 3), "GBps": round(wl.bytes / ev_us / 1e3, 1),
+                         "frac_of_hbm_peak": round(wl.bytes / ev_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "note": "the GEMV kernel with its weight, activation, scale and zero loads and no arithmetic"}
+    if timeline:
+        n_waves = plan["workgroups"] * waves
+        trace = torch.zeros((n_waves, 5), dtype=torch.int64, device=wl.y.device)
+        rows = []
+        for i in range(40):
+            trace.zero_()
+            torch.cuda.synchronize()
+            # behind a few ordinary launches, so that the probe launch meets the queue as a timed step does
+            for w in range(3):
+                wl.launch(i + w)
+            j = (i + 3) % wl.sets
+            mg.probe_gemv(mg.PROBE_TIMELINE, trace, wl.w[j], wl.x, wl.s[j], wl.z[j], wl.y, wl.n_out, wl.k, wl.group)
+            torch.cuda.synchronize()
+            t = trace.cpu().numpy().astype("float64")
+            t = t[t[:, 0] > 0]
+            if len(t) == 0:
+                continue
+            t0 = t[:, 0].min()
+            med = lambda v: float(statistics.median(v))  # noqa: E731
+            rows.append([med(t[:, 0] - t0), float((t[:, 0] - t0).max()), med(t[:, 1] - t[:, 0]), med(t[:, 2] - t[:, 1]),
+                         med(t[:, 3] - t[:, 2]), med(t[:, 4] - t[:, 3]), float(t[:, 4].max() - t0)])
+        if rows:
+            tick_us = 0.01  # s_memrealtime counts a constant 100 MHz clock
+            col = lambda c: round(statistics.median(r[c] for r in rows[5:] or rows) * tick_us, 3)  # noqa: E731
+            out["timeline_us"] = {
+                "clock": "s_memrealtime, 100 MHz (10 ns per tick); medians over the waves of a launch, then over launches",
+                "wave_start_after_first_wave_median": col(0), "wave_start_after_first_wave_last": col(1),
+                "start_to_first_unit_requested": col(2), "requested_to_first_block_arrived": col(3),
+                "first_block_to_last_unit_computed": col(4), "last_unit_to_outputs_stored": col(5),
+                "first_wave_start_to_last_store": col(6), "waves": n_waves, "launches": len(rows)}
+    return out
 
 
 def _oracle_operands(wl, j):
@@ -446,6 +514,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and every oracle check")
     ap.add_argument("--no-warm-cache", action="store_true",
                     help="skip the warm-cache and launch-floor side measurements (keeps a kernel trace to the cold launches)")
+    ap.add_argument("--no-ceilings", action="store_true",
+                    help="skip the ceiling measurements (plain streaming reads, the kernel without its arithmetic, "
+                         "the timeline of one launch)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy 512 MiB device to device four times and exit: the known-size kernel against which "
                          "the FETCH_SIZE / WRITE_SIZE counters of `rocprofv3 --pmc` are scaled")
@@ -525,11 +596,12 @@ def main():
         wl.sets = all_sets
         out["warm_cache"] = {"us_per_call": w["us_per_call"], "GBps": w["value_GBps"],
                              "note": "one buffer set re-read from the 256 MB Infinity Cache; not an HBM figure"}
-        if use_graph:
-            floor = launch_floor_us(device)
-            out["launch_floor"] = {"us_per_launch": round(floor, 3),
-                                   "kernel_us_above_floor": round(kernel_us - floor, 3),
-                                   "note": "graph replay of a one-element fill kernel: the cadence of an empty launch"}
+        floor = launch_floor_us(use_graph)
+        out["launch_floor"] = {"us_per_launch": round(floor, 3),
+                               "kernel_us_above_floor": round(kernel_us - floor, 3),
+                               "note": "cadence of an empty kernel (mgemv_probe_empty_launch) launched like the timed steps"}
+    if not args.no_ceilings:
+        out["ceilings"] = {wl.name: ceilings_of(wl, use_graph, timeline=True)}
     if not args.no_cpu:
         cpu = cpu_baseline(wl)
         out["cpu_baseline"] = {
@@ -576,6 +648,8 @@ def main():
             # config 5 names 8 distinct rotated buffers: all of them are checked, not only the first
             sets = list(range(w2.sets)) if base == "c5" else [0]
             entry["parity"] = parity_summary(w2, sets, threads, with_dequant=(rows in (None, 1)))
+        if base == "c5" and element == "f16" and batch == 1 and not args.no_ceilings:
+            out.setdefault("ceilings", {})[base] = ceilings_of(w2, use_graph)
         others[name] = entry
     built.clear()
     torch.cuda.empty_cache()

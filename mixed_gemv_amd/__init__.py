@@ -16,6 +16,11 @@ from .api import (  # noqa: F401
     device_gemv,
     gemv_arguments,
     host_gemv,
+    probe_empty_launch,
+    probe_gemv,
+    probe_stream_read,
+    PROBE_LOADS_ONLY,
+    PROBE_TIMELINE,
     preprocessed_size,
     query_launch,
     set_launch_override,

@@ -41,6 +41,9 @@ SIGNATURES = {
     "mgemv_query_launch_bf16": (_c.c_int, [_c.c_int] * 5 + [_c.POINTER(_c.c_int * 8)]),
     "mgemv_query_launch_for": (_c.c_int, [_c.c_int] * 7 + [_c.POINTER(_c.c_int * 8)]),
     "mgemv_gemv_arguments": (_c.c_int, [_vp, _vp]),
+    "mgemv_probe_empty_launch": (_c.c_int, [_vp]),
+    "mgemv_probe_stream_read": (_c.c_int, [_vp, _c.c_size_t, _c.c_int, _c.c_int, _c.c_int, _vp, _vp]),
+    "mgemv_probe_gemv": (_c.c_int, [_c.c_int, _vp, _vp, _u16p, _u16p, _u16p, _u16p, _c.c_int, _c.c_int, _c.c_int, _vp]),
     "mgemv_host_gemv": (_c.c_int, [_c.c_int] * 5 + [_vp] * 6 + [_c.c_int] * 2),
     "mgemv_tuned_plan_set": (_c.c_int, [_c.POINTER(_c.c_int * 10)]),
     "mgemv_tuned_plan_clear": (_c.c_int, []),

@@ -330,6 +330,30 @@ def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0, element="f16", 
     return dict(zip(keys, list(out)))
 
 
+PROBE_LOADS_ONLY = 1
+PROBE_TIMELINE = 2
+
+
+def probe_empty_launch(stream=None):
+    """One empty kernel launch (mgemv_probe_empty_launch)."""
+    _lib.check(_lib.lib().mgemv_probe_empty_launch(_stream_ptr(stream)), "probe_empty_launch")
+
+
+def probe_stream_read(src, nbytes, workgroups, waves_per_workgroup, units_in_flight, sink=None, stream=None):
+    """Plain streaming read of nbytes at src with the GEMV's weight loads (mgemv_probe_stream_read)."""
+    _lib.check(_lib.lib().mgemv_probe_stream_read(_dev_ptr(src), int(nbytes), int(workgroups), int(waves_per_workgroup),
+                                                  int(units_in_flight), _dev_ptr(sink), _stream_ptr(stream)),
+               "probe_stream_read")
+
+
+def probe_gemv(kind, trace, ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_D, M, K, group_size, stream=None):
+    """Measurement builds of the headline kernel (mgemv_probe_gemv): PROBE_LOADS_ONLY or PROBE_TIMELINE
+    (trace: int64 device tensor of 5 entries per wave)."""
+    _lib.check(_lib.lib().mgemv_probe_gemv(int(kind), _dev_ptr(trace), _dev_ptr(ptr_A), _dev_ptr(ptr_B),
+                                           _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_D), int(M), int(K),
+                                           int(group_size), _stream_ptr(stream)), "probe_gemv")
+
+
 KERNEL_AUTO = 0
 KERNEL_VALU = 1
 KERNEL_MATRIX_CORE_REGISTER_OPERAND = 2

@@ -14,7 +14,8 @@ LIB_PATH = os.path.join(LIB_DIR, "libmixed_gemv_amd.so")
 LINT_REPORT = os.path.join(LIB_DIR, "isa_lint.json")
 
 # One translation unit per family of kernel instantiations, so that they compile side by side.
-SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "gemv_kernels.hip", "host_utils.cpp"]
+SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "gemv_kernels.hip", "probes.hip",
+           "host_utils.cpp"]
 
 # -ffp-contract=off: the dequantiser is a separately rounded fp16 multiply and add.
 # -packed-fp32-ops off: keep the compiler from forming v_pk_*_f32.

@@ -246,9 +246,25 @@ __device__ __forceinline__ void compute_unit_form(float (&acc)[MB], const UnitFr
 }
 
 // short_allowed: wave-uniform.
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, int ACT = kActF16>
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, int ACT = kActF16, int PROBE = kProbeNone>
 __device__ __forceinline__ void compute_unit(float (&acc)[MB], const UnitFragment<BITS, MB, GROUPS_PER_RUN>& f,
                                              const ConvertRegs& c, bool short_allowed) {
+  if constexpr (PROBE == kProbeLoadsOnly) {
+    // every register of the unit has to arrive, nothing is computed
+    uint32_t t = 0;
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) t ^= f.s[gi] ^ (QOP == MGEMV_FINEGRAINED_SCALE_AND_ZEROS ? f.z[gi] : 0u);
+#pragma unroll
+    for (int i = 0; i < kBlocksPerUnit; ++i) t ^= f.w[i][0] ^ f.w[i][1] ^ f.w[i][2] ^ f.w[i][3];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) {
+      uint32_t tm = t;
+#pragma unroll
+      for (int h = 0; h < (BITS == 4 ? 4 : 2); ++h) tm ^= f.x[m][h];
+      acc[m] += __builtin_bit_cast(float, tm & 0x3fffffffu);
+    }
+    return;
+  }
   if constexpr (BITS == 4 || ACT == kActBf16) {
     if (short_allowed && wave_scales_permit_short_form<ACT>(f.s)) {
       compute_unit_form<BITS, QOP, MB, GROUPS_PER_RUN, true, ACT>(acc, f, c);
@@ -294,12 +310,18 @@ __device__ __forceinline__ void finish_tile(float (&acc)[MB], float* slot) {
 // The allocation unit is 8 registers, so 81 would already cost a whole wave of occupancy.
 // ACT: kActF16 or kActBf16 -- the type of activations, scales, zeros, bias and outputs (the
 // pointers are typed as 16-bit storage either way).
-template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI, int ACT>
+// PROBE (measurement builds of this same kernel, see mixed_gemv.h "Measurement probes"):
+// kProbeNone the product; kProbeLoadsOnly keeps every load and replaces the arithmetic of a unit
+// by an exclusive-or over its registers -- what the access pattern alone takes; kProbeTimeline
+// records five timestamps per wave.
+template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI, int ACT, int PROBE = kProbeNone>
 __global__ void __launch_bounds__(kWave * (MB >= 3 || ACT == kActBf16 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
 __attribute__((amdgpu_waves_per_eu(ACT == kActF16 && MB == 1 && GROUPS_PER_RUN == 1 ? 6 : 1)))
 gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out, int k,
                 uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
   extern __shared__ float partials[];
+  uint64_t stamp[5] = {0, 0, 0, 0, 0};
+  if constexpr (PROBE == kProbeTimeline) stamp[0] = __builtin_amdgcn_s_memrealtime();
   Problem p;
   p.weights = weights;
   p.x = x;
@@ -380,6 +402,13 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     // fragments inside, without that wait, measured the same to 2 % on every shape.)
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
     load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
+    if constexpr (PROBE == kProbeTimeline) {
+      __builtin_amdgcn_sched_barrier(0);
+      stamp[1] = __builtin_amdgcn_s_memrealtime();      // the first unit is requested
+      asm volatile("s_waitcnt vmcnt(3)" ::: "memory");   // ... and all but its last three blocks are in
+      stamp[2] = __builtin_amdgcn_s_memrealtime();
+      __builtin_amdgcn_sched_barrier(0);
+    }
     const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
     const ConvertRegs c = make_convert_regs();
     // With two or more activation rows, a wave of exactly two units runs straight-line code: the
@@ -389,15 +418,15 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     // single-row kernels, which are held to 80 registers, any extra path made the loop beside it
     // 4-7 % slower, so those keep the loop for every length.
     if (total == 1) {
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
       if constexpr (MULTI) finish_tile<MB>(acc, slot);
     } else if (MB >= 2 && !MULTI && total == 2) {
       advance<MULTI>(cur, walk);
       load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
       __builtin_amdgcn_sched_barrier(0);
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
       __builtin_amdgcn_sched_barrier(0);
-      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fb, c, short_ok);
+      compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fb, c, short_ok);
     } else {
       // The prefetches are unconditional: past the wave's last unit every weight offset is out
       // of the descriptor's range, the loads return zero without touching memory, and the
@@ -407,7 +436,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         advance<MULTI>(cur, walk);
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
         __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
-        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fa, c, short_ok);
+        compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
         if constexpr (MULTI) {
           if (--pending == 0) {
             finish_tile<MB>(acc, slot);
@@ -419,7 +448,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
         __builtin_amdgcn_sched_barrier(0);
         if (u + 1 < total) {
-          compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT>(acc, fb, c, short_ok);
+          compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fb, c, short_ok);
           if constexpr (MULTI) {
             if (--pending == 0) {
               finish_tile<MB>(acc, slot);
@@ -430,6 +459,12 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         __builtin_amdgcn_sched_barrier(0);
         u += 2;
       } while (u < total);
+    }
+    if constexpr (PROBE == kProbeTimeline) {
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("" :: "v"(acc[0]));
+      stamp[3] = __builtin_amdgcn_s_memrealtime();      // the last unit is computed
+      __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!MULTI) finish_tile<MB>(acc, partials + (ty * split_k + kw) * MB * kWave + lane_after_loop());
   }
@@ -453,6 +488,15 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     }
     for (; w < split_k; ++w) sum += part[w * MB * kWave];
     store_outputs<ACT>(tail, has_bias, p.n_out, m, tile_begin + j, lane_c, reduce_k_slices(sum));
+  }
+  if constexpr (PROBE == kProbeTimeline) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // the outputs are on their way
+    stamp[4] = __builtin_amdgcn_s_memrealtime();
+    if (tail.trace != nullptr && lane_c == 0) {
+      unsigned long long* out = tail.trace + ((size_t)blockIdx.x * (blockDim.x * blockDim.y / kWave) + ty * split_k + kw) * 5;
+#pragma unroll
+      for (int i = 0; i < 5; ++i) out[i] = stamp[i];
+    }
   }
 }
 

@@ -477,7 +477,8 @@ PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_ba
 int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
              const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k, int group_size,
              int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
-             int64_t stride_bias, int64_t stride_y, void* stream, int act, float alpha = 1.0f, float beta = 1.0f) {
+             int64_t stride_bias, int64_t stride_y, void* stream, int act, float alpha = 1.0f, float beta = 1.0f,
+             int probe = kProbeNone, unsigned long long* trace = nullptr) {
   if (batch_count < 1 || batch_count > 65535) return MGEMV_ERR_BATCH;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
@@ -507,6 +508,7 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
   g.tail.flags = g_dequant_flags.load();
   g.tail.alpha = alpha;
   g.tail.beta = beta;
+  g.tail.trace = trace;
   {
     const int sequences = g.plan.workgroups * g.plan.tiles_per_wg;
     g.tail.seq_base = num_tiles(n_out) / sequences;
@@ -537,6 +539,15 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
     g.lds = g.plan.split_k == 1 ? 0
                                 : (size_t)g.plan.tiles_per_wg * g.plan.split_k * g.plan.tiles_per_wave * kWave * 4 * sizeof(float);
     return launch_mfma(g, weight_bits, quant_op, gpr) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+  }
+  if (probe != kProbeNone) {
+    // measurement builds exist for the headline kernel only: int4, scale and zero, one group per run, one row, fp16
+    if (weight_bits != 4 || quant_op != MGEMV_FINEGRAINED_SCALE_AND_ZEROS || gpr != 1 || m_batch != 1 || act != kActF16)
+      return MGEMV_ERR_QUANT_OP;
+    g.x = reinterpret_cast<const half_t*>(x);
+    g.tail.y = reinterpret_cast<half_t*>(y);
+    g.lds = (size_t)g.plan.tiles_in_sequence * g.plan.tiles_per_wg * g.plan.split_k * kWave * sizeof(float);
+    return launch_gemv_probe(g, probe) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
   }
   // VALU path: activation rows are processed kMaxValuBatch at a time.
   for (int m0 = 0; m0 < m_batch; m0 += kMaxValuBatch) {
@@ -624,6 +635,15 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
                      int k, int group_size, int quant_op, int weight_bits, void* stream) {
   return mgemv::dequantize_any(weights, scale, zero_add, out, n_out, k, group_size, quant_op, weight_bits, stream,
                                mgemv::kActF16);
+}
+
+int mgemv_probe_gemv(int kind, unsigned long long* trace, const void* weights, const uint16_t* x, const uint16_t* scale,
+                     const uint16_t* zero_add, uint16_t* y, int n_out, int k, int group_size, void* stream) {
+  if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_TIMELINE) return MGEMV_ERR_SIZE;
+  if (kind == MGEMV_PROBE_TIMELINE && (trace == nullptr || reinterpret_cast<uintptr_t>(trace) % 8)) return MGEMV_ERR_NULL_POINTER;
+  return mgemv::gemv_any(weights, x, scale, zero_add, nullptr, y, 1, n_out, 1, k, group_size,
+                         MGEMV_FINEGRAINED_SCALE_AND_ZEROS, 4, 0, 0, 0, 0, 0, stream, mgemv::kActF16, 1.0f, 1.0f,
+                         kind == MGEMV_PROBE_LOADS_ONLY ? mgemv::kProbeLoadsOnly : mgemv::kProbeTimeline, trace);
 }
 
 // gemv/device/gemv_adaptor.h:114-178 as one plain struct.

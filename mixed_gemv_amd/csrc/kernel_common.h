@@ -19,6 +19,7 @@ constexpr int kNumXcd = 8;
 constexpr int kNumCus = 256;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
+constexpr int kProbeNone = 0, kProbeLoadsOnly = 1, kProbeTimeline = 2;  // measurement builds of the VALU kernel
 
 // Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are what a
 // wave needs to address its first loads, and they are preloaded into SGPRs (build flag
@@ -34,6 +35,7 @@ struct GemvTail {
   int seq_base;        // VALU kernel: tiles / sequences ...
   int seq_rem;         // ... and tiles % sequences (the first seq_rem sequences get one tile more)
   long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
+  unsigned long long* trace;  // timeline probe: five timestamps per wave, else unused
 };
 
 // Scalar view of one problem inside a kernel.
@@ -172,6 +174,8 @@ hipError_t launch_gemv_f16(const GemvLaunch& g, int bits, int qop, int mb, int g
 hipError_t launch_gemv_bf16(const GemvLaunch& g, int bits, int qop, int mb, int gpr);
 hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr);
 hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act);
+// Measurement builds of the single-row int4 scale-and-zero fp16 VALU kernel (probe: kProbeLoadsOnly / kProbeTimeline).
+hipError_t launch_gemv_probe(const GemvLaunch& g, int probe);
 
 }  // namespace mgemv
 

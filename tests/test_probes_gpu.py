@@ -1,0 +1,53 @@
+"""The measurement probes of the library (include/mixed_gemv.h, "Measurement probes"): they run,
+the timeline build of the kernel still computes the GEMV, and its timestamps are ordered."""
+import numpy as np
+import pytest
+
+import mixed_gemv_amd as mg
+from helpers import SCALE_AND_ZEROS, DeviceProblem, Problem
+from mixed_gemv_amd._lib import MixedGemvError
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("n_out,k,cap", [(512, 4096, 0), (4096, 2048, 0), (192, 8192, 5)])  # cap: waves walk several tiles
+def test_timeline_build_is_the_product_kernel_plus_timestamps(gpu, n_out, k, cap):
+    import torch
+    prob = Problem("probe", n_out, k, 4, SCALE_AND_ZEROS, 128, x_dist="normal")
+    dev = DeviceProblem(prob, gpu)
+    try:
+        mg.set_launch_override(0, 0, 0, cap)
+        want = dev.run().copy()
+        plan = mg.query_launch(n_out, 1, k, 4, 128)
+        waves = plan["workgroups"] * plan["threads"] // 64
+        trace = torch.zeros((waves, 5), dtype=torch.int64, device=gpu)
+        dev.y.fill_(0x7e00)
+        mg.probe_gemv(mg.PROBE_TIMELINE, trace, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 128)
+        torch.cuda.synchronize()
+        assert np.array_equal(dev.y.cpu().numpy().view(np.uint16), want.view(np.uint16))
+        t = trace.cpu().numpy()
+        t = t[t[:, 0] > 0]                                  # workgroups past the last tile leave before stamping
+        assert len(t) >= (n_out // 16) * plan["split_k"] // max(plan["tiles_in_sequence"], 1) // 2
+        assert np.all(np.diff(t, axis=1) >= 0)              # entry <= requested <= arrived <= computed <= stored
+        assert (t[:, 4] - t[:, 0]).max() < 100_000          # 10 ns ticks: under a millisecond
+        mg.probe_gemv(mg.PROBE_LOADS_ONLY, None, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 128)
+        torch.cuda.synchronize()
+    finally:
+        mg.set_launch_override(0, 0, 0, 0)
+
+
+def test_stream_read_and_empty_launch_run_and_check_their_arguments(gpu):
+    import torch
+    buf = torch.zeros(8 << 20, dtype=torch.uint8, device=gpu)
+    sink = torch.zeros(1, dtype=torch.int32, device=gpu)
+    for wgs, waves, depth in ((256, 4, 2), (64, 16, 4), (8, 1, 8)):
+        mg.probe_stream_read(buf, buf.numel(), wgs, waves, depth, sink)
+    mg.probe_empty_launch()
+    torch.cuda.synchronize()
+    for bad in ((0, 4, 2), (256, 17, 2), (256, 4, 3), (4096, 16, 2)):   # the last: less than one unit per wave
+        with pytest.raises(MixedGemvError):
+            mg.probe_stream_read(buf, buf.numel(), *bad, sink)
+    with pytest.raises(MixedGemvError):
+        mg.probe_gemv(mg.PROBE_TIMELINE, None, buf, buf, buf, buf, buf, 64, 512, 128)   # needs a trace buffer
+    with pytest.raises(MixedGemvError):
+        mg.probe_gemv(mg.PROBE_LOADS_ONLY, None, buf, buf, buf, buf, buf, 64, 512, 64)  # two groups per run: no probe build
