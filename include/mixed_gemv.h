@@ -243,6 +243,14 @@ MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 enum { MGEMV_MATRIX_CORE_AUTO = 0, MGEMV_MATRIX_CORE_REGISTER_OPERAND = 1, MGEMV_MATRIX_CORE_LDS_STAGED = 2 };
 MGEMV_API int mgemv_set_matrix_core_variant(int variant);
 
+/* The reference's kStages (mixed_gemv_test.cu:40; gemv/threadblock/default_dq_mma_simt.h:224-234 for
+ * the single-stage main loop, :394-404 for the two-stage one) for the VALU kernel: 2 keeps the
+ * loads of the next 16-row x 512-k unit in flight while a unit is computed, 1 waits for every load
+ * before it computes (loads and arithmetic strictly one after the other), 0 restores the built-in
+ * choice (2).  Same results either way.  The matrix-core kernels always run two stages.  For
+ * tuning and tests.  Process-wide. */
+MGEMV_API int mgemv_set_prefetch_stages(int stages);
+
 /* Which int4 dequantiser the kernels may use.  Both produce the same bits, rn16(rn16(q*s) + z)
  * as gemv/warp/warp_dequantizer.h:52-59:
  *   MGEMV_DEQUANT_AUTO (default)    per wave and k step, the one-FMA form wherever every scale
@@ -288,10 +296,10 @@ MGEMV_API int mgemv_fold_zero_points_bf16(uint16_t *out, const uint16_t *scales,
  * matches every group size (an entry for the exact group size wins); per-column problems are
  * looked up with group_size = k.  The knobs have the meaning of mgemv_set_launch_override
  * (0 = built-in rule for that knob); `kernel` picks the kernel.  A process-wide override that is
- * set (mgemv_set_launch_override, _matrix_core_threshold, _matrix_core_variant) takes precedence
+ * set (mgemv_set_launch_override, _matrix_core_threshold, _matrix_core_variant, _prefetch_stages) takes precedence
  * over the table.  Setting an existing key replaces it.  Results never depend on the plan beyond
- * the order of the fp32 partial sums.  The fp16 and the _bf16 entry points share the table (a bf16
- * launch clamps an entry to what its kernels allow).  Thread-safe. */
+ * the order of the fp32 partial sums.  An entry serves launches of its own element type only (a
+ * bf16 launch clamps an entry to what its kernels allow).  Thread-safe. */
 enum {
   MGEMV_KERNEL_AUTO = 0,
   MGEMV_KERNEL_VALU = 1,
@@ -302,8 +310,12 @@ typedef struct mgemv_tuned_plan {
   int n_out, k, weight_bits, group_size, m_batch; /* key */
   int kernel;                                     /* MGEMV_KERNEL_* */
   int split_k_waves, tiles_per_workgroup, tiles_per_wave, max_workgroups;
+  int stages;                                     /* 0 built-in, 1 or 2: see mgemv_set_prefetch_stages */
+  int element;                                    /* key: MGEMV_ELEMENT_F16 / MGEMV_ELEMENT_BF16 launches only */
 } mgemv_tuned_plan;
 MGEMV_API int mgemv_tuned_plan_set(const mgemv_tuned_plan *plan);
+/* Removes the entry with exactly plan's key fields, if there is one (the other fields are not read). */
+MGEMV_API int mgemv_tuned_plan_erase(const mgemv_tuned_plan *plan);
 MGEMV_API int mgemv_tuned_plan_clear(void);
 MGEMV_API int mgemv_tuned_plan_count(void);
 
@@ -322,9 +334,25 @@ MGEMV_API int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits,
  * the matrix-core kernels only the LDS-staged one exists for bf16). */
 MGEMV_API int mgemv_query_launch_bf16(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]);
 /* The same for either element type (MGEMV_ELEMENT_*) and a device of num_compute_units compute
- * units (a partition of an MI355X has 32 per XCD). */
+ * units (a partition of an MI355X has 32 per XCD), plus what the plan asks of the hardware:
+ * out[8] = bytes of dynamic LDS per workgroup, out[9] = the workgroup size limit the chosen
+ * kernel is compiled for, out[10] = prefetch stages (1 or 2), out[11] = launches that serve all
+ * activation rows (the VALU kernel takes four rows per launch). */
 MGEMV_API int mgemv_query_launch_for(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
-                                     int num_compute_units, int out[8]);
+                                     int num_compute_units, int out[12]);
+
+/* Replays, on the host, the index arithmetic every wave of that launch would do -- the same
+ * functions the kernels are compiled from -- and reports whether the plan covers the problem:
+ * the counterpart of checking the reference's grid (gemv/device/gemv_adaptor.h:190-197) against
+ * its threadblock tile offsets (gemv/kernel/mixed_gemv.h:134-139).  Needs no GPU.
+ * out[0] = tiles (16 output rows) whose k steps are not covered exactly once (must be 0),
+ * out[1] = waves whose range leaves the problem or that have no k step, duplicate workgroups (0),
+ * out[2] = most bytes behind one wave's weight descriptor (< 2^31),
+ * out[3] = VALU kernel: bytes of LDS up to the last partial sum any wave parks (<= out[4]),
+ * out[4] = bytes of dynamic LDS the launch asks for, out[5] = waves with work,
+ * out[6] = launched waves without a tile, out[7] = most 16-row x k-step units one wave computes. */
+MGEMV_API int mgemv_plan_coverage(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
+                                  int num_compute_units, int64_t out[8]);
 
 /* ------------------------------------------------------------------------------------------
  * Measurement probes.  No counterpart in the reference and not on any product path: they are

@@ -22,10 +22,12 @@ from .api import (  # noqa: F401
     PROBE_LOADS_ONLY,
     PROBE_TIMELINE,
     preprocessed_size,
+    plan_coverage,
     query_launch,
     set_launch_override,
     set_matrix_core_threshold,
     set_dequant_form,
+    set_prefetch_stages,
     set_matrix_core_variant,
     MATRIX_CORE_AUTO,
     MATRIX_CORE_REGISTER_OPERAND,
@@ -33,6 +35,7 @@ from .api import (  # noqa: F401
     DEQUANT_AUTO,
     DEQUANT_EXACT_INTEGER,
     unpreprocess_weights,
+    erase_tuned_plan,
     set_tuned_plan,
     clear_tuned_plans,
     tuned_plan_count,

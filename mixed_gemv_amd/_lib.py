@@ -39,13 +39,16 @@ SIGNATURES = {
     "mgemv_set_matrix_core_variant": (_c.c_int, [_c.c_int]),
     "mgemv_query_launch": (_c.c_int, [_c.c_int] * 5 + [_c.POINTER(_c.c_int * 8)]),
     "mgemv_query_launch_bf16": (_c.c_int, [_c.c_int] * 5 + [_c.POINTER(_c.c_int * 8)]),
-    "mgemv_query_launch_for": (_c.c_int, [_c.c_int] * 7 + [_c.POINTER(_c.c_int * 8)]),
+    "mgemv_query_launch_for": (_c.c_int, [_c.c_int] * 7 + [_c.POINTER(_c.c_int * 12)]),
+    "mgemv_set_prefetch_stages": (_c.c_int, [_c.c_int]),
+    "mgemv_plan_coverage": (_c.c_int, [_c.c_int] * 7 + [_c.POINTER(_c.c_int64 * 8)]),
     "mgemv_gemv_arguments": (_c.c_int, [_vp, _vp]),
     "mgemv_probe_empty_launch": (_c.c_int, [_vp]),
     "mgemv_probe_stream_read": (_c.c_int, [_vp, _c.c_size_t, _c.c_int, _c.c_int, _c.c_int, _vp, _vp]),
     "mgemv_probe_gemv": (_c.c_int, [_c.c_int, _vp, _vp, _u16p, _u16p, _u16p, _u16p, _c.c_int, _c.c_int, _c.c_int, _vp]),
     "mgemv_host_gemv": (_c.c_int, [_c.c_int] * 5 + [_vp] * 6 + [_c.c_int] * 2),
-    "mgemv_tuned_plan_set": (_c.c_int, [_c.POINTER(_c.c_int * 10)]),
+    "mgemv_tuned_plan_set": (_c.c_int, [_c.POINTER(_c.c_int * 12)]),
+    "mgemv_tuned_plan_erase": (_c.c_int, [_c.POINTER(_c.c_int * 12)]),
     "mgemv_tuned_plan_clear": (_c.c_int, []),
     "mgemv_tuned_plan_count": (_c.c_int, []),
 }

@@ -316,18 +316,36 @@ def query_launch(n_out, m_batch, k, weight_bits=4, group_size=0, element="f16", 
     """The geometry mgemv_gemv (element="bf16": mgemv_gemv_bf16) would use on an unpartitioned MI355X, or on
     a device of num_compute_units compute units; group_size as passed to the GEMV (it only selects tuned
     plans)."""
-    out = (ctypes.c_int * 8)()
-    if num_compute_units is not None:
-        _lib.check(_lib.lib().mgemv_query_launch_for(int(n_out), int(m_batch), int(k), int(weight_bits),
-                                                     int(group_size), 1 if _is_bf16(element, None) else 0,
-                                                     int(num_compute_units), ctypes.byref(out)), "query_launch")
-    else:
+    if num_compute_units is None:
+        out = (ctypes.c_int * 8)()
         fn = _lib.lib().mgemv_query_launch_bf16 if _is_bf16(element, None) else _lib.lib().mgemv_query_launch
         _lib.check(fn(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size), ctypes.byref(out)),
                    "query_launch")
+    else:
+        out = (ctypes.c_int * 12)()
+        _lib.check(_lib.lib().mgemv_query_launch_for(int(n_out), int(m_batch), int(k), int(weight_bits),
+                                                     int(group_size), 1 if _is_bf16(element, None) else 0,
+                                                     int(num_compute_units), ctypes.byref(out)), "query_launch")
     keys = ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "matrix_core", "tiles_per_wave",
-            "tiles_in_sequence")
+            "tiles_in_sequence", "lds_bytes", "max_threads", "stages", "launches")
     return dict(zip(keys, list(out)))
+
+
+def plan_coverage(n_out, m_batch, k, weight_bits=4, group_size=0, element="f16", num_compute_units=256):
+    """Host replay of every wave's index arithmetic for the launch plan of this problem (mgemv_plan_coverage)."""
+    out = (ctypes.c_int64 * 8)()
+    _lib.check(_lib.lib().mgemv_plan_coverage(int(n_out), int(m_batch), int(k), int(weight_bits), int(group_size),
+                                              1 if _is_bf16(element, None) else 0, int(num_compute_units),
+                                              ctypes.byref(out)), "plan_coverage")
+    keys = ("tiles_miscovered", "bad_waves", "max_descriptor_bytes", "lds_bytes_used", "lds_bytes", "busy_waves",
+            "idle_waves", "max_units_per_wave")
+    return dict(zip(keys, list(out)))
+
+
+def set_prefetch_stages(stages):
+    """1: the VALU kernel waits for every load before it computes; 2: the next unit's loads are in flight
+    meanwhile; 0: built-in choice (mgemv_set_prefetch_stages)."""
+    _lib.check(_lib.lib().mgemv_set_prefetch_stages(int(stages)), "set_prefetch_stages")
 
 
 PROBE_LOADS_ONLY = 1
@@ -361,11 +379,20 @@ KERNEL_MATRIX_CORE_LDS_STAGED = 3
 
 
 def set_tuned_plan(n_out, k, weight_bits, group_size, m_batch, kernel=KERNEL_AUTO, split_k=0, tiles_per_wg=0,
-                   tiles_per_wave=0, max_workgroups=0):
-    """Installs the launch plan for exactly this problem; see mgemv_tuned_plan_set (group_size 0 = any)."""
-    plan = (ctypes.c_int * 10)(int(n_out), int(k), int(weight_bits), int(group_size), int(m_batch), int(kernel),
-                               int(split_k), int(tiles_per_wg), int(tiles_per_wave), int(max_workgroups))
+                   tiles_per_wave=0, max_workgroups=0, stages=0, element="f16"):
+    """Installs the launch plan for exactly this problem and element type; see mgemv_tuned_plan_set
+    (group_size 0 = any)."""
+    plan = (ctypes.c_int * 12)(int(n_out), int(k), int(weight_bits), int(group_size), int(m_batch), int(kernel),
+                               int(split_k), int(tiles_per_wg), int(tiles_per_wave), int(max_workgroups), int(stages),
+                               1 if _is_bf16(element, None) else 0)
     _lib.check(_lib.lib().mgemv_tuned_plan_set(ctypes.byref(plan)), "set_tuned_plan")
+
+
+def erase_tuned_plan(n_out, k, weight_bits, group_size, m_batch, element="f16"):
+    """Removes the table entry of exactly this key, if any (mgemv_tuned_plan_erase)."""
+    plan = (ctypes.c_int * 12)(int(n_out), int(k), int(weight_bits), int(group_size), int(m_batch), 0, 0, 0, 0, 0, 0,
+                               1 if _is_bf16(element, None) else 0)
+    _lib.check(_lib.lib().mgemv_tuned_plan_erase(ctypes.byref(plan)), "erase_tuned_plan")
 
 
 def clear_tuned_plans():

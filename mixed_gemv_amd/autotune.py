@@ -27,7 +27,7 @@ _installed = {}  # key tuple -> entry dict, what save_table writes
 def candidate_plans(n_out, k, weight_bits, m_batch):
     """Knob settings worth measuring, as dicts for set_tuned_plan (duplicates in effect are
     removed later by comparing the geometry the library reports)."""
-    out = [dict(kernel=api.KERNEL_AUTO)]
+    out = [dict(kernel=api.KERNEL_AUTO), dict(kernel=api.KERNEL_AUTO, stages=1)]
     wave_limit = 8 if m_batch >= 3 else 16
     for tiles_per_wg in (1, 2, 4):
         for split_k in (1, 2, 4, 8, 16):
@@ -100,9 +100,15 @@ class _Problem:
         return e0.elapsed_time(e1) * 1e3 / (replays * nodes)
 
 
-def _key(n_out, k, weight_bits, quant_op, group_size, m_batch):
+def _key(n_out, k, weight_bits, quant_op, group_size, m_batch, element="f16"):
     per_column = int(quant_op) == int(api.WeightOnlyQuantOp.PER_COLUMN_SCALE_ONLY)
-    return (int(n_out), int(k), int(weight_bits), int(k if per_column else group_size), int(m_batch))
+    return (int(n_out), int(k), int(weight_bits), int(k if per_column else group_size), int(m_batch),
+            "bf16" if element == "bf16" else "f16")
+
+
+def _entry_key(entry):
+    return (entry["n_out"], entry["k"], entry["weight_bits"], entry["group_size"], entry["m_batch"],
+            entry.get("element", "f16"))
 
 
 def install(entry):
@@ -110,19 +116,31 @@ def install(entry):
     api.set_tuned_plan(entry["n_out"], entry["k"], entry["weight_bits"], entry["group_size"], entry["m_batch"],
                        kernel=entry.get("kernel", 0), split_k=entry.get("split_k", 0),
                        tiles_per_wg=entry.get("tiles_per_wg", 0), tiles_per_wave=entry.get("tiles_per_wave", 0),
-                       max_workgroups=entry.get("max_workgroups", 0))
-    _installed[(entry["n_out"], entry["k"], entry["weight_bits"], entry["group_size"], entry["m_batch"])] = dict(entry)
+                       max_workgroups=entry.get("max_workgroups", 0), stages=entry.get("stages", 0),
+                       element=entry.get("element", "f16"))
+    _installed[_entry_key(entry)] = dict(entry)
+
+
+def erase(key):
+    """Removes the entry of one key (n_out, k, weight_bits, group_size, m_batch, element) from the
+    library's table and from what save_table writes."""
+    api.erase_tuned_plan(*key[:5], element=key[5])
+    _installed.pop(key, None)
 
 
 def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, group_size=128,
          m_batch=1, bias=False, device="cuda:0", launches=400, rounds=2, min_gain=0.02, seed=1,
          cold_bytes=_CACHE_BYTES, log=None, element="f16"):
     """Measures the candidate plans for this problem and installs the fastest, unless it beats the
-    built-in plan by less than `min_gain` (then the table is left alone for this key).  Returns a
+    built-in plan by less than `min_gain` (then the key ends up without an entry: one left by an
+    earlier run is removed, since the built-in plan has just been measured to be as good).  Every
+    candidate, the built-in plan included, is measured with a process-wide override set, which
+    makes the library ignore the table, so an entry that already exists never stands in for the
+    built-in plan.  Returns a
     dict with the chosen entry (or None), the built-in time and every measurement.  `cold_bytes`
     is how much operand data is rotated between two uses of the same buffers (default: more than
-    the Infinity Cache).  `element` ("f16" / "bf16") picks the entry points that are timed; the table
-    itself is shared by both, so tune for the element type the process will run.
+    the Infinity Cache).  `element` ("f16" / "bf16") picks the entry points that are timed; an entry
+    serves launches of its own element type only.
 
     Must not run while other threads launch GEMVs: the candidates are applied through the
     process-wide overrides."""
@@ -130,7 +148,8 @@ def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCA
     if not torch.cuda.is_available():
         raise RuntimeError("autotune.tune needs the GPU")
     device = torch.device(device)
-    key = _key(n_out, k, weight_bits, quant_op, group_size, m_batch)
+    key = _key(n_out, k, weight_bits, quant_op, group_size, m_batch, element)
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
     prob = _Problem(n_out, k, weight_bits, api.WeightOnlyQuantOp(quant_op), key[3], m_batch, bias, device, seed,
                     cold_bytes, element)
     seen, results = {}, []
@@ -142,7 +161,8 @@ def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCA
                 prob.time_us(launches)
             for cand in candidate_plans(n_out, k, weight_bits, m_batch):
                 _apply(cand)
-                geometry = tuple(sorted(api.query_launch(n_out, m_batch, k, weight_bits, key[3], element=element).items()))
+                geometry = tuple(sorted(api.query_launch(n_out, m_batch, k, weight_bits, key[3], element=element,
+                                                         num_compute_units=cus).items()))
                 if geometry in seen:
                     continue
                 seen[geometry] = cand
@@ -161,20 +181,25 @@ def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCA
                     best_us = min(best_us, prob.time_us(launches))
     finally:
         _apply(dict(kernel=api.KERNEL_AUTO))
+        api.set_prefetch_stages(0)
     entry = None
     if best is not results[0][1] and best_us < builtin_us * (1.0 - min_gain):
         entry = dict(n_out=key[0], k=key[1], weight_bits=key[2], group_size=key[3], m_batch=key[4],
                      kernel=best.get("kernel", 0), split_k=best.get("split_k", 0),
                      tiles_per_wg=best.get("tiles_per_wg", 0), tiles_per_wave=best.get("tiles_per_wave", 0),
-                     max_workgroups=best.get("max_workgroups", 0), us=round(best_us, 3),
-                     builtin_us=round(builtin_us, 3))
+                     max_workgroups=best.get("max_workgroups", 0), stages=best.get("stages", 0), element=key[5],
+                     us=round(best_us, 3), builtin_us=round(builtin_us, 3))
         install(entry)
+    else:
+        erase(key)
     return dict(entry=entry, builtin_us=builtin_us, best_us=best_us, best_geometry=best_geometry,
+                builtin_geometry=results[0][2],
                 measurements=[(us, _describe(c)) for us, c, _ in results])
 
 
 def _apply(cand):
     kernel = cand.get("kernel", api.KERNEL_AUTO)
+    api.set_prefetch_stages(cand.get("stages", 2))  # 2 is the built-in value; any override set bypasses the table
     api.set_launch_override(cand.get("split_k", 0), cand.get("tiles_per_wg", 0), cand.get("tiles_per_wave", 0),
                             cand.get("max_workgroups", 0))
     api.set_matrix_core_threshold({api.KERNEL_AUTO: 0, api.KERNEL_VALU: 17}.get(kernel, 1))

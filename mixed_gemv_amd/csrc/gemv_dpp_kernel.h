@@ -360,16 +360,10 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);         // tile sequence within the workgroup
   const int split_k = tail.split_k;
   const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
-  // The tiles are dealt out evenly, in contiguous runs, to the (workgroups x tiles_per_wg) tile
-  // sequences of the launch; the split_k waves of a sequence walk its tiles together, each on
-  // its own part of k.
-  const int seq = wg * p.tiles_per_wg + ty;
-  const int tile_begin = MULTI ? seq * tail.seq_base + min(seq, tail.seq_rem) : seq;
-  const int my_tiles = MULTI ? tail.seq_base + (seq < tail.seq_rem ? 1 : 0) : (seq < tiles ? 1 : 0);
-
   // The host's launch geometry leaves no wave without units (split_k = ceil(ksteps / steps_per_wave)).
-  const int ks_begin = kw * p.steps_per_wave;
-  const int units = min(ks_begin + p.steps_per_wave, p.ksteps) - ks_begin;
+  const WaveWork work = valu_wave_work(MULTI, wg, ty, kw, p.tiles_per_wg, tail.seq_base, tail.seq_rem, tiles,
+                                       p.steps_per_wave, p.ksteps);
+  const int tile_begin = work.tile_begin, my_tiles = work.tiles, ks_begin = work.ks_begin, units = work.units;
   const int park_stride = p.tiles_per_wg * split_k * MB * kWave;  // floats between consecutive tiles of a sequence
 
   if (my_tiles > 0) {
@@ -431,10 +425,17 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       // The prefetches are unconditional: past the wave's last unit every weight offset is out
       // of the descriptor's range, the loads return zero without touching memory, and the
       // compiler can count outstanding loads exactly instead of draining them all before each use.
+      // The reference's kStages = 1 main loop (gemv/threadblock/dq_mma_singlestage_finegrained.h:264-310)
+      // keeps nothing in flight while it computes; its kStages = 2 loop (dq_mma_pipelined_finegrained.h:
+      // 263-352) is this one.  With the single-stage flag every prefetch is waited for as soon as it is
+      // issued, which gives that behaviour -- loads and arithmetic strictly one after the other -- to the
+      // same code; results do not change.
+      const bool single_stage = (tail.flags & kSingleStage) != 0;
       int u = 0;
       do {
         advance<MULTI>(cur, walk);
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
+        if (single_stage) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
         compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
         if constexpr (MULTI) {
@@ -446,6 +447,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         advance<MULTI>(cur, walk);
         __builtin_amdgcn_sched_barrier(0);
         load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
+        if (single_stage) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         if (u + 1 < total) {
           compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fb, c, short_ok);

@@ -119,6 +119,7 @@ std::atomic<int> g_override_tiles_per_wave{0};
 std::atomic<int> g_override_workgroups{0};
 std::atomic<int> g_matrix_core_min_batch{0};  // m_batch from which the matrix-core kernels are used; 0 = built-in rule
 std::atomic<int> g_dequant_flags{0};          // kExactIntegerFormOnly or 0
+std::atomic<int> g_override_stages{0};        // 0 = built-in (2), 1 or 2
 std::atomic<int> g_matrix_core_variant{MGEMV_MATRIX_CORE_AUTO};
 
 // What steers plan_launch besides the shape: zeros mean "built-in rule".
@@ -127,18 +128,19 @@ struct PlanKnobs {
   int matrix_core_min_batch = 0;
   int matrix_core_variant = MGEMV_MATRIX_CORE_AUTO;
   bool wide_waves = false;  // the kernel is one of those compiled for at most 8 waves per workgroup
+  int stages = 0;           // VALU kernel: 0 = built-in rule (2: the next unit in flight while one is computed), 1, 2
   int num_cus = kNumCus;    // compute units of the device the launch goes to (256 on an unpartitioned MI355X)
 };
 
 // Tuned plans by problem: (n_out, k, weight bits, group size or 0 for any, m_batch) -> knobs.
-using PlanKey = std::tuple<int, int, int, int, int>;
+using PlanKey = std::tuple<int, int, int, int, int, int>;  // n_out, k, bits, group size, rows, element
 std::mutex g_tuned_mutex;
 std::map<PlanKey, PlanKnobs> g_tuned_plans;
 std::atomic<int> g_tuned_count{0};  // lets the launch path skip the lock while the table is empty
 
 // Process-wide overrides win over the table (they are what a tuner sweeps); then an entry for
 // exactly this group size, then one for any group size, then the built-in rules.
-PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
+PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch, int act) {
   PlanKnobs kn;
   kn.split_k = g_override_split_k.load();
   kn.tiles_per_wg = g_override_tiles_per_wg.load();
@@ -146,12 +148,14 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch) {
   kn.workgroups = g_override_workgroups.load();
   kn.matrix_core_min_batch = g_matrix_core_min_batch.load();
   kn.matrix_core_variant = g_matrix_core_variant.load();
-  const bool overridden = kn.split_k || kn.tiles_per_wg || kn.tiles_per_wave || kn.workgroups ||
+  kn.stages = g_override_stages.load();
+  const bool overridden = kn.split_k || kn.tiles_per_wg || kn.tiles_per_wave || kn.workgroups || kn.stages ||
                           kn.matrix_core_min_batch || kn.matrix_core_variant != MGEMV_MATRIX_CORE_AUTO;
   if (overridden || g_tuned_count.load() == 0) return kn;
   std::lock_guard<std::mutex> lock(g_tuned_mutex);
-  auto it = g_tuned_plans.find(PlanKey{n_out, k, bits, group_size, m_batch});
-  if (it == g_tuned_plans.end() && group_size != 0) it = g_tuned_plans.find(PlanKey{n_out, k, bits, 0, m_batch});
+  const int element = act == kActBf16 ? MGEMV_ELEMENT_BF16 : MGEMV_ELEMENT_F16;
+  auto it = g_tuned_plans.find(PlanKey{n_out, k, bits, group_size, m_batch, element});
+  if (it == g_tuned_plans.end() && group_size != 0) it = g_tuned_plans.find(PlanKey{n_out, k, bits, 0, m_batch, element});
   return it == g_tuned_plans.end() ? kn : it->second;
 }
 
@@ -186,7 +190,7 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs& knobs) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
-  const int cus = knobs.num_cus > 0 ? knobs.num_cus : cus;  // the thresholds below were measured on 256 and scale with it
+  const int cus = knobs.num_cus > 0 ? knobs.num_cus : kNumCus;  // the thresholds below were measured on 256 and scale with it
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
   const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves, bits, cus);
@@ -249,6 +253,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     lp.threads = kWave * lp.split_k * lp.tiles_per_wg;
     lp.tiles_per_wave = 1;
     lp.tiles_in_sequence = 1;
+    lp.stages = 2;
     return lp;
   }
   // Matrix-core path: a wave that works on T tiles fetches the activation operands of a k step
@@ -358,6 +363,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   lp.tiles_in_sequence = 1;
   lp.staged_rows = 0;
   lp.matrix_core = mc;
+  lp.stages = !mc && knobs.stages == 1 ? 1 : 2;
   if (!mc) {
     // VALU path: fewer workgroups than tile groups means every wave walks several tiles.
     const int ov_wg = knobs.workgroups;
@@ -414,6 +420,34 @@ int groups_per_run(int group_size, int bits) {
   return group_size % run == 0 ? 1 : 2;
 }
 
+// What a plan asks of the hardware: dynamic LDS of its (largest) launch, the workgroup size limit the
+// kernel it picks was compiled for, and how many launches serve all activation rows.
+struct LaunchResources {
+  size_t lds_bytes;
+  int max_threads;
+  int launches;
+};
+LaunchResources launch_resources(const LaunchPlan& lp, int bits, int m_batch, int act) {
+  LaunchResources r{};
+  r.launches = 1;
+  if (lp.matrix_core) {
+    r.max_threads = kWave * kMaxWavesPerMfmaWorkgroup;
+    if (lp.staged_rows != 0) {
+      const int row_stride = step_k(bits) * 2 + 16;
+      r.lds_bytes = (size_t)lp.split_k * 2 * lp.staged_rows * row_stride +
+                    (lp.split_k > 1 ? (size_t)lp.tiles_per_wg * lp.split_k * kWave * 4 * sizeof(float) : 0);
+    } else {
+      r.lds_bytes = lp.split_k == 1 ? 0 : (size_t)lp.tiles_per_wg * lp.split_k * lp.tiles_per_wave * kWave * 4 * sizeof(float);
+    }
+    return r;
+  }
+  const int rows = m_batch < kMaxValuBatch ? m_batch : kMaxValuBatch;
+  r.launches = (m_batch + kMaxValuBatch - 1) / kMaxValuBatch;
+  r.max_threads = kWave * (rows >= 3 || act == kActBf16 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup);
+  r.lds_bytes = (size_t)lp.tiles_in_sequence * lp.tiles_per_wg * lp.split_k * rows * kWave * sizeof(float);
+  return r;
+}
+
 hipError_t launch_gemv(const GemvLaunch& g, int bits, int qop, int mb, int gpr, int act) {
   return act == kActBf16 ? launch_gemv_bf16(g, bits, qop, mb, gpr) : launch_gemv_f16(g, bits, qop, mb, gpr);
 }
@@ -461,7 +495,7 @@ int device_info(int device, DeviceInfo& info) {
 
 // The knobs of a problem with the element type taken into account.
 PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_batch, int act, int num_cus = kNumCus) {
-  PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch);
+  PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch, act);
   knobs.num_cus = num_cus;
   if (act == kActBf16) {
     // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
@@ -505,7 +539,7 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
-  g.tail.flags = g_dequant_flags.load();
+  g.tail.flags = g_dequant_flags.load() | (g.plan.stages == 1 ? kSingleStage : 0);
   g.tail.alpha = alpha;
   g.tail.beta = beta;
   g.tail.trace = trace;
@@ -528,16 +562,12 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
     g.x = reinterpret_cast<const half_t*>(x);
     g.tail.y = reinterpret_cast<half_t*>(y);
     g.tail.m_batch = m_batch;
+    g.lds = launch_resources(g.plan, weight_bits, m_batch, act).lds_bytes;
     if (g.plan.staged_rows != 0) {
-      const int row_stride = step_k(weight_bits) * 2 + 16;
-      g.lds = (size_t)g.plan.split_k * 2 * g.plan.staged_rows * row_stride +
-              (g.plan.split_k > 1 ? (size_t)g.plan.tiles_per_wg * g.plan.split_k * kWave * 4 * sizeof(float) : 0);
       return launch_mfma_lds(g, weight_bits, quant_op, gpr, g.plan.staged_rows / g.plan.tiles_per_wg, act) == hipSuccess
                  ? MGEMV_OK
                  : MGEMV_ERR_LAUNCH;
     }
-    g.lds = g.plan.split_k == 1 ? 0
-                                : (size_t)g.plan.tiles_per_wg * g.plan.split_k * g.plan.tiles_per_wave * kWave * 4 * sizeof(float);
     return launch_mfma(g, weight_bits, quant_op, gpr) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
   }
   if (probe != kProbeNone) {
@@ -746,6 +776,12 @@ int mgemv_set_matrix_core_variant(int variant) {
   return MGEMV_OK;
 }
 
+int mgemv_set_prefetch_stages(int stages) {
+  if (stages < 0 || stages > 2) return MGEMV_ERR_SIZE;
+  mgemv::g_override_stages.store(stages);
+  return MGEMV_OK;
+}
+
 int mgemv_set_dequant_form(int form) {
   if (form != MGEMV_DEQUANT_AUTO && form != MGEMV_DEQUANT_EXACT_INTEGER) return MGEMV_ERR_SIZE;
   mgemv::g_dequant_flags.store(form == MGEMV_DEQUANT_EXACT_INTEGER ? mgemv::kExactIntegerFormOnly : 0);
@@ -767,6 +803,8 @@ int mgemv_tuned_plan_set(const mgemv_tuned_plan* plan) {
   const int st = check_tuned_key(plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch);
   if (st != MGEMV_OK) return st;
   if (plan->split_k_waves < 0 || plan->tiles_per_workgroup < 0 || plan->max_workgroups < 0) return MGEMV_ERR_SIZE;
+  if (plan->stages < 0 || plan->stages > 2) return MGEMV_ERR_SIZE;
+  if (plan->element != MGEMV_ELEMENT_F16 && plan->element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
   const int t = plan->tiles_per_wave;
   if (t != 0 && t != 1 && t != 2 && t != 4) return MGEMV_ERR_SIZE;
   mgemv::PlanKnobs kn;
@@ -774,6 +812,7 @@ int mgemv_tuned_plan_set(const mgemv_tuned_plan* plan) {
   kn.tiles_per_wg = plan->tiles_per_workgroup;
   kn.tiles_per_wave = t;
   kn.workgroups = plan->max_workgroups;
+  kn.stages = plan->stages;
   switch (plan->kernel) {
     case MGEMV_KERNEL_AUTO: break;
     case MGEMV_KERNEL_VALU: kn.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1; break;
@@ -788,7 +827,17 @@ int mgemv_tuned_plan_set(const mgemv_tuned_plan* plan) {
     default: return MGEMV_ERR_SIZE;
   }
   std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);
-  mgemv::g_tuned_plans[mgemv::PlanKey{plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch}] = kn;
+  mgemv::g_tuned_plans[mgemv::PlanKey{plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch,
+                                      plan->element}] = kn;
+  mgemv::g_tuned_count.store((int)mgemv::g_tuned_plans.size());
+  return MGEMV_OK;
+}
+
+int mgemv_tuned_plan_erase(const mgemv_tuned_plan* plan) {
+  if (plan == nullptr) return MGEMV_ERR_NULL_POINTER;
+  std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);
+  mgemv::g_tuned_plans.erase(
+      mgemv::PlanKey{plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch, plan->element});
   mgemv::g_tuned_count.store((int)mgemv::g_tuned_plans.size());
   return MGEMV_OK;
 }
@@ -808,11 +857,91 @@ int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_s
 }
 
 int mgemv_query_launch_for(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
-                           int num_compute_units, int out[8]) {
+                           int num_compute_units, int out[12]) {
   if (element != MGEMV_ELEMENT_F16 && element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
   if (num_compute_units < 1 || num_compute_units > 4096) return MGEMV_ERR_SIZE;
-  return query_launch_any(n_out, m_batch, k, weight_bits, group_size,
-                          element == MGEMV_ELEMENT_BF16 ? mgemv::kActBf16 : mgemv::kActF16, out, num_compute_units);
+  const int act = element == MGEMV_ELEMENT_BF16 ? mgemv::kActBf16 : mgemv::kActF16;
+  if (const int st = query_launch_any(n_out, m_batch, k, weight_bits, group_size, act, out, num_compute_units)) return st;
+  const mgemv::LaunchPlan lp = mgemv::plan_launch(
+      n_out, k, weight_bits, m_batch, mgemv::knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act, num_compute_units));
+  const mgemv::LaunchResources r = mgemv::launch_resources(lp, weight_bits, m_batch, act);
+  out[8] = (int)r.lds_bytes;
+  out[9] = r.max_threads;
+  out[10] = lp.stages;
+  out[11] = r.launches;
+  return MGEMV_OK;
+}
+
+int mgemv_plan_coverage(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
+                        int num_compute_units, int64_t out[8]) {
+  using namespace mgemv;
+  if (out == nullptr) return MGEMV_ERR_NULL_POINTER;
+  if (element != MGEMV_ELEMENT_F16 && element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
+  if (num_compute_units < 1 || num_compute_units > 4096) return MGEMV_ERR_SIZE;
+  if (const int st = check_tuned_key(n_out, k, weight_bits, group_size, m_batch)) return st;
+  const int act = element == MGEMV_ELEMENT_BF16 ? kActBf16 : kActF16;
+  const LaunchPlan lp = plan_launch(n_out, k, weight_bits, m_batch,
+                                    knobs_for_element(n_out, k, weight_bits, group_size, m_batch, act, num_compute_units));
+  const LaunchResources res = launch_resources(lp, weight_bits, m_batch, act);
+  const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, weight_bits);
+  const int grid = lp.wgs_per_xcd * kNumXcd;
+  const int sequences = lp.workgroups * lp.tiles_per_wg;
+  const int seq_base = tiles / sequences, seq_rem = tiles % sequences;  // as gemv_any passes them
+  const bool multi = !lp.matrix_core && lp.tiles_in_sequence > 1;
+  const int rows = m_batch < kMaxValuBatch ? m_batch : kMaxValuBatch;
+  std::vector<int> covered((size_t)tiles, 0);
+  std::vector<char> block_seen((size_t)lp.workgroups, 0);
+  int64_t idle_waves = 0, busy_waves = 0, max_span = 0, max_lds = 0, bad_ranges = 0, max_units = 0;
+  for (int block = 0; block < grid; ++block) {
+    const int wg = logical_workgroup_of(block, lp.wgs_per_xcd);
+    if (wg >= lp.workgroups) continue;  // the kernels leave at this test
+    if (block_seen[(size_t)wg]++) ++bad_ranges;   // two blocks with one logical id
+    for (int ty = 0; ty < lp.tiles_per_wg; ++ty) {
+      for (int kw = 0; kw < lp.split_k; ++kw) {
+        const WaveWork w = lp.matrix_core
+                               ? (lp.staged_rows != 0
+                                      ? staged_wave_work(wg, ty, kw, lp.tiles_per_wg, tiles, lp.steps_per_wave, ksteps)
+                                      : mfma_wave_work(lp.tiles_per_wave, wg, ty, kw, lp.tiles_per_wg, tiles,
+                                                       lp.steps_per_wave, ksteps))
+                               : valu_wave_work(multi, wg, ty, kw, lp.tiles_per_wg, seq_base, seq_rem, tiles,
+                                                lp.steps_per_wave, ksteps);
+        if (w.units <= 0) ++bad_ranges;  // every kernel relies on each wave along k having units
+        if (w.tiles <= 0 || w.units <= 0) {
+          ++idle_waves;
+          continue;
+        }
+        ++busy_waves;
+        if (w.tile_begin < 0 || w.tile_begin + w.tiles > tiles || w.ks_begin < 0 || w.ks_begin + w.units > ksteps) {
+          ++bad_ranges;
+          continue;
+        }
+        for (int t = 0; t < w.tiles; ++t) covered[(size_t)(w.tile_begin + t)] += w.units;
+        // the bytes one weight descriptor spans: tiles are ksteps units apart
+        const int64_t span = (int64_t)(w.tiles - 1) * ksteps * kUnitBytes + (int64_t)w.units * kUnitBytes;
+        max_span = span > max_span ? span : max_span;
+        const int64_t walk_units = (int64_t)w.tiles * w.units;
+        max_units = walk_units > max_units ? walk_units : max_units;
+        if (!lp.matrix_core) {
+          // last float this wave parks for the combine (tile t of its walk at t * park_stride)
+          const int64_t park_stride = (int64_t)lp.tiles_per_wg * lp.split_k * rows * kWave;
+          const int64_t last = (int64_t)(multi ? w.tiles - 1 : 0) * park_stride +
+                               ((int64_t)(ty * lp.split_k + kw) * rows + (rows - 1)) * kWave + (kWave - 1);
+          max_lds = (last + 1) * 4 > max_lds ? (last + 1) * 4 : max_lds;
+        }
+      }
+    }
+  }
+  int64_t wrong = 0;
+  for (int t = 0; t < tiles; ++t) wrong += covered[(size_t)t] != ksteps;
+  out[0] = wrong;                 // tiles whose k steps are not covered exactly once
+  out[1] = bad_ranges;            // waves with a range outside the problem or without units, duplicate workgroup ids
+  out[2] = max_span;              // most bytes behind one weight descriptor
+  out[3] = max_lds;               // VALU kernel: bytes of LDS up to the last parked partial sum
+  out[4] = (int64_t)res.lds_bytes;
+  out[5] = busy_waves;
+  out[6] = idle_waves;
+  out[7] = max_units;             // most units any wave computes
+  return MGEMV_OK;
 }
 
 int mgemv_query_launch(int n_out, int m_batch, int k, int weight_bits, int group_size, int out[8]) {

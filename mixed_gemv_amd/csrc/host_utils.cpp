@@ -301,6 +301,6 @@ const char* mgemv_status_string(int status) {
   }
 }
 
-int mgemv_version(void) { return 210; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
+int mgemv_version(void) { return 211; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
 
 }  // extern "C"

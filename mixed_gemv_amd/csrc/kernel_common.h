@@ -19,6 +19,7 @@ constexpr int kNumXcd = 8;
 constexpr int kNumCus = 256;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
+constexpr int kSingleStage = 2;           // GemvTail::flags: no load in flight while a unit is computed (VALU kernel)
 constexpr int kProbeNone = 0, kProbeLoadsOnly = 1, kProbeTimeline = 2;  // measurement builds of the VALU kernel
 
 // Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are what a
@@ -30,7 +31,7 @@ struct GemvTail {
   int split_k;         // waves of a workgroup that share one tile (blockDim.x / 64)
   int m_batch;         // activation rows (matrix-core kernel)
   int num_groups;      // k / group_size (1 in per-column mode): extent of the scale / zero tables
-  int flags;           // kExactIntegerFormOnly or 0
+  int flags;           // kExactIntegerFormOnly | kSingleStage
   float alpha, beta;   // epilogue: y = alpha * acc + beta * bias (gemv/device/gemv_adaptor.h:123, epilogue{alpha, beta})
   int seq_base;        // VALU kernel: tiles / sequences ...
   int seq_rem;         // ... and tiles % sequences (the first seq_rem sequences get one tile more)
@@ -57,13 +58,72 @@ struct Problem {
 constexpr uint32_t pack_steps(int ksteps, int steps_per_wave) { return (uint32_t)ksteps | ((uint32_t)steps_per_wave << 16); }
 constexpr uint32_t pack_group(int group_size, int tiles_per_wg) { return (uint32_t)group_size | ((uint32_t)tiles_per_wg << 24); }
 
+// ---------------------------------------------------------------------------------------------
+// Which part of the problem a wave works on.  Plain integer functions, compiled for the device
+// (the kernels call them) and for the host (which replays them over a whole grid to check that a
+// launch plan covers every tile and k step exactly once).
+// ---------------------------------------------------------------------------------------------
+
 // Workgroups are handed to the 8 XCDs round-robin by linear id.  Neighbouring tiles read
 // neighbouring 32-byte pieces of the same scale/zero cache lines, so give each XCD (and its
 // private L2) a contiguous range of tiles instead of every eighth one.
+__host__ __device__ __forceinline__ int logical_workgroup_of(int block, int wgs_per_xcd) {
+  const int xcd = block % kNumXcd;
+  const int slot = block / kNumXcd;
+  return xcd * wgs_per_xcd + slot;
+}
+
+struct WaveWork {
+  int tile_begin, tiles;  // tiles tile_begin .. tile_begin + tiles - 1 (tiles may be 0)
+  int ks_begin, units;    // k steps ks_begin .. ks_begin + units - 1 of each of them (units may be <= 0)
+};
+
+// k range of the kw-th wave along k.
+__host__ __device__ __forceinline__ void wave_k_range(WaveWork& w, int kw, int steps_per_wave, int ksteps) {
+  w.ks_begin = kw * steps_per_wave;
+  const int end = w.ks_begin + steps_per_wave < ksteps ? w.ks_begin + steps_per_wave : ksteps;
+  w.units = end - w.ks_begin;
+}
+
+// VALU kernel.  The tiles are dealt out evenly, in contiguous runs, to the (workgroups x
+// tiles_per_wg) tile sequences of the launch (multi: sequence s takes seq_base tiles, the first
+// seq_rem sequences one more); the split_k waves of a sequence walk its tiles together, each on
+// its own part of k.  Without walks (multi false) sequence s is tile s.
+__host__ __device__ __forceinline__ WaveWork valu_wave_work(bool multi, int wg, int ty, int kw, int tiles_per_wg,
+                                                            int seq_base, int seq_rem, int tiles, int steps_per_wave,
+                                                            int ksteps) {
+  WaveWork w;
+  const int seq = wg * tiles_per_wg + ty;
+  w.tile_begin = multi ? seq * seq_base + (seq < seq_rem ? seq : seq_rem) : seq;
+  w.tiles = multi ? seq_base + (seq < seq_rem ? 1 : 0) : (seq < tiles ? 1 : 0);
+  wave_k_range(w, kw, steps_per_wave, ksteps);
+  return w;
+}
+
+// Register-operand matrix-core kernel: a wave takes tiles_per_wave consecutive tiles.
+__host__ __device__ __forceinline__ WaveWork mfma_wave_work(int tiles_per_wave, int wg, int ty, int kw, int tiles_per_wg,
+                                                            int tiles, int steps_per_wave, int ksteps) {
+  WaveWork w;
+  w.tile_begin = (wg * tiles_per_wg + ty) * tiles_per_wave;
+  const int left = tiles - w.tile_begin;
+  w.tiles = left <= 0 ? 0 : left < tiles_per_wave ? left : tiles_per_wave;
+  wave_k_range(w, kw, steps_per_wave, ksteps);
+  return w;
+}
+
+// LDS-staged matrix-core kernel: one tile per wave; a wave past the last tile has no tile of
+// its own (it still stages activation rows and meets the barriers).
+__host__ __device__ __forceinline__ WaveWork staged_wave_work(int wg, int ty, int kw, int tiles_per_wg, int tiles,
+                                                              int steps_per_wave, int ksteps) {
+  WaveWork w;
+  w.tile_begin = wg * tiles_per_wg + ty;
+  w.tiles = w.tile_begin < tiles ? 1 : 0;
+  wave_k_range(w, kw, steps_per_wave, ksteps);
+  return w;
+}
+
 __device__ __forceinline__ int logical_workgroup(const Problem& p) {
-  const int xcd = blockIdx.x % kNumXcd;
-  const int slot = blockIdx.x / kNumXcd;
-  return xcd * p.wgs_per_xcd + slot;
+  return logical_workgroup_of((int)blockIdx.x, p.wgs_per_xcd);
 }
 
 // Group index of reduction position k_index (host/mixed_gemv.h:88), clamped to the last
@@ -142,6 +202,7 @@ struct LaunchPlan {
   int tiles_per_wave;  // 1 on the VALU path; 1, 2 or 4 on the matrix-core path
   int tiles_in_sequence;  // VALU path: most tiles any wave walks one after the other
   int staged_rows;        // LDS-staged matrix-core kernel: 8 or 16 activation rows per stage; 0 = other kernels
+  int stages;             // VALU path: 2 = the next unit is in flight while one is computed, 1 = it is not
   bool matrix_core;       // one of the two matrix-core kernels (else the VALU kernel)
 };
 

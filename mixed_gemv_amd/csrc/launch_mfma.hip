@@ -234,8 +234,9 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   const int lane = threadIdx.x % kWave;
   const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);
-  const int tile0 = (wg * p.tiles_per_wg + ty) * T;
   const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
+  const WaveWork work = mfma_wave_work(T, wg, ty, kw, p.tiles_per_wg, tiles, p.steps_per_wave, p.ksteps);
+  const int tile0 = work.tile_begin;
   int row[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) {
@@ -246,11 +247,10 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   f32x4 acc[T];
 #pragma unroll
   for (int t = 0; t < T; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-  const int ks_begin = kw * p.steps_per_wave;
-  const int ks_end = min(ks_begin + p.steps_per_wave, p.ksteps);
-  if (tile0 < tiles && ks_begin < ks_end) {
-    const int units = ks_end - ks_begin;
-    const int my_tiles = min(T, tiles - tile0);
+  const int ks_begin = work.ks_begin;
+  if (work.tiles > 0 && work.units > 0) {
+    const int units = work.units;
+    const int my_tiles = work.tiles;
     const int tile_stride = p.ksteps * kUnitBytes;  // bytes from a unit to the same k step of the next tile
     // One descriptor spans the wave's tiles.
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
@@ -456,8 +456,9 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
   const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);
   const int split_k = tail.split_k;
   const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
-  const int tile_raw = wg * p.tiles_per_wg + ty;
-  const int tile = tile_raw < tiles ? tile_raw : tiles - 1;  // a wave without a tile still stages rows and meets the barriers
+  const WaveWork work = staged_wave_work(wg, ty, kw, p.tiles_per_wg, tiles, p.steps_per_wave, p.ksteps);
+  const int tile_raw = work.tile_begin;
+  const int tile = work.tiles > 0 ? tile_raw : tiles - 1;  // a wave without a tile still stages rows and meets the barriers
   const int row_raw = tile * kTileRows + lane % kTileRows;
   const int row = row_raw < p.n_out ? row_raw : p.n_out - 1;
 
@@ -470,8 +471,8 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
   const int operand_offset = m_read * XS::kRowStride + (lane / kTileRows) * Geometry<BITS>::kRunK * 2;
 
   const int steps = p.steps_per_wave;  // the same for every wave: the barriers are workgroup-wide
-  const int ks_begin = kw * steps;
-  const int units = min(ks_begin + steps, p.ksteps) - ks_begin;  // >= 1 by the host's geometry
+  const int ks_begin = work.ks_begin;
+  const int units = work.units;  // >= 1 by the host's geometry
   const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(
       p.weights + ((size_t)tile * (size_t)p.ksteps + (size_t)ks_begin) * (size_t)kUnitBytes,
       (uint32_t)units * (uint32_t)kUnitBytes);

@@ -271,22 +271,57 @@ def test_tuner_measures_installs_and_keeps_parity(gpu, m_batch):
     prob = Problem("tuner", 1024, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=m_batch, bias=True)
     autotune.clear()
     try:
-        before = mg.query_launch(1024, m_batch, 2048, 4, 128)
+        cus = 256
+        before = mg.query_launch(1024, m_batch, 2048, 4, 128, num_compute_units=cus)
+        # an entry left by an earlier run (a poor one) must neither pass for the built-in plan nor survive
+        mg.set_tuned_plan(1024, 2048, 4, 128, m_batch, kernel=mg.KERNEL_VALU, split_k=1, tiles_per_wg=1, max_workgroups=1)
+        assert mg.query_launch(1024, m_batch, 2048, 4, 128, num_compute_units=cus) != before
         lines = []
         res = autotune.tune(1024, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=m_batch, bias=True, launches=64, rounds=1,
                             min_gain=0.0, cold_bytes=8 << 20, log=lines.append)
         print("\n".join(lines), flush=True)
         assert len(res["measurements"]) >= 4 and all(us > 0 for us, _ in res["measurements"])
         assert res["entry"] is None or res["entry"]["us"] < res["entry"]["builtin_us"]
-        after = mg.query_launch(1024, m_batch, 2048, 4, 128)
+        assert res["builtin_geometry"] == before
+        after = mg.query_launch(1024, m_batch, 2048, 4, 128, num_compute_units=cus)
         if res["entry"] is None:
             assert after == before and mg.tuned_plan_count() == 0
         else:
-            assert after == res["best_geometry"] and mg.tuned_plan_count() == 1
+            assert after == res["best_geometry"] and mg.tuned_plan_count() == 1 and res["entry"]["element"] == "f16"
         assert mg.query_launch(2048, m_batch, 2048, 4, 128) == mg.query_launch(2048, m_batch, 2048, 4, 0)
         check(prob, gpu, dequant=False)
     finally:
         autotune.clear()
+
+
+@pytest.mark.parametrize("tag,n_out,k,bits,qop,g,m_batch,cap", [
+    ("st_ns", 4096, 4096, 4, SCALE_AND_ZEROS, 128, 1, 0),        # four waves of two units
+    ("st_walk", 1024, 8192, 4, SCALE_AND_ZEROS, 128, 1, 8),      # walks of eight tiles
+    ("st_rows", 512, 6144, 4, SCALE_ONLY, 64, 3, 0),
+    ("st_i8", 768, 4096, 8, PER_COLUMN, 0, 2, 5),
+    ("st_bf16", 640, 5120, 4, SCALE_AND_ZEROS, 128, 1, 3),
+])
+def test_single_stage_loop_gives_the_same_bits(gpu, tag, n_out, k, bits, qop, g, m_batch, cap):
+    """kStages = 1 against 2 (gemv/threadblock/default_dq_mma_simt.h:224-234, 394-404): the same
+    arithmetic in the same order, only without a load in flight beside it."""
+    prob = Problem(tag, n_out, k, bits, qop, g, m_batch=m_batch, bias=True, x_dist="normal",
+                   element="bf16" if tag.endswith("bf16") else "f16")
+    dev = DeviceProblem(prob, gpu)
+    try:
+        mg.set_launch_override(0, 0, 0, cap)
+        mg.set_matrix_core_threshold(17)
+        two = dev.run().copy()
+        mg.set_prefetch_stages(1)
+        assert mg.query_launch(n_out, m_batch, k, bits, g, element=prob.element, num_compute_units=256)["stages"] == 1
+        one = dev.run().copy()
+    finally:
+        mg.set_prefetch_stages(0)
+        mg.set_matrix_core_threshold(0)
+        mg.set_launch_override(0, 0, 0, 0)
+    assert np.array_equal(one.view(np.uint16), two.view(np.uint16))
+    if prob.element == "f16":   # (the bf16 two-stage result is pinned to the oracle by the bf16 tests)
+        _, rel, _ = error_report(one, prob.oracle_gemv(threads=8))
+        assert rel <= REL_TOL
 
 
 WALKS = [
