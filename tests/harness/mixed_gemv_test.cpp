@@ -109,6 +109,24 @@ int main(int argc, char** argv) {
   HIP_CHECK(hipDeviceSynchronize());
   HIP_CHECK(hipGetLastError());
 
+  // The reference's HOST_CHECK call site (mixed_gemv_test.cu:167-181) with the GPU behind it:
+  // un-preprocessed weights and int8 zero points in, result out.  Same kernels on the same
+  // values, so it must reproduce the device result bit for bit.
+  std::vector<half_t> h_D_call_site((size_t)B * M * kGemmN);
+  try {
+    host_gemv(reinterpret_cast<const uint8_t*>(h_A.data()), h_B.data(), h_scale.data(), h_zero_point.data(),
+              with_bias ? h_bias.data() : nullptr, h_D_call_site.data(), B, M, kGemmN, K, group_size, quant_op, bits);
+  } catch (const Error& e) {
+    std::printf("host_gemv: %s\n", e.what());
+    return 4;
+  }
+  size_t call_site_diffs = 0;
+  for (size_t i = 0; i < result_D.size(); ++i) call_site_diffs += h_D_call_site[i] != result_D[i];
+  if (call_site_diffs) {
+    std::printf("host::reference::MixedGemv differs from device_gemv in %zu outputs\n", call_site_diffs);
+    return 5;
+  }
+
   // HOST_CHECK: un-preprocessed weights, int8 zero points (host/mixed_gemv.h:60-105)
   std::vector<half_t> h_D((size_t)B * M * kGemmN);
   orc_gemv(h_D.data(), h_A.data(), h_B.data(), h_scale.data(), h_zero_point.data(), with_bias ? h_bias.data() : nullptr,
