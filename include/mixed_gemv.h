@@ -57,7 +57,8 @@ typedef enum mgemv_status {
                                    the batch strides to match); scales, zeros, bias, outputs 2 bytes; the output of
                                    mgemv_dequantize 4 bytes */
   MGEMV_ERR_LEADING_DIMENSION = 14, /* mgemv_gemv_arguments: a leading dimension other than the dense one */
-  MGEMV_ERR_ALLOCATION = 15     /* mgemv_host_gemv: device memory could not be allocated */
+  MGEMV_ERR_ALLOCATION = 15,    /* mgemv_host_gemv: device memory could not be allocated */
+  MGEMV_ERR_SCRATCH_SIZE = 16   /* mgemv_host_gemv_static: the problem needs more than MGEMV_STATIC_SCRATCH_BYTES */
 } mgemv_status;
 
 /* gemv/weight_only_quant_op.h:12-18 — same numeric values. */
@@ -206,6 +207,27 @@ MGEMV_API int mgemv_gemv_arguments(const mgemv_arguments *args, void *stream);
 MGEMV_API int mgemv_host_gemv(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t *weights,
                               const uint16_t *x, const uint16_t *scale, const int8_t *zero_point,
                               const uint16_t *bias, uint16_t *y, int quant_op, int weight_bits);
+
+/* mgemv_host_gemv without any allocation.  It has no counterpart in the reference; it is for
+ * callers that cannot allocate device memory where they call from -- harnesses that forbid
+ * hipMalloc, tight serving loops -- and still want the HOST_CHECK-shaped call.  Same arguments,
+ * same results bit for bit.  The device staging that mgemv_host_gemv allocates per call
+ * (preprocessed weights, folded zeros, activations, tables, bias, outputs; 256-byte aligned
+ * pieces) lives in a static device array of MGEMV_STATIC_SCRATCH_BYTES that every GPU the library
+ * runs on holds until the process ends, and the host-side temporaries in a static host array of
+ * the same size: no hipMalloc, hipFree or heap allocation on this path.  A problem whose pieces do
+ * not fit returns MGEMV_ERR_SCRATCH_SIZE (mgemv_static_scratch_bytes_needed tells beforehand).
+ * All calls in a process share the arrays (each GPU its own device copy, all of them the one
+ * host array) and are serialised by a lock inside the library; the arrays keep the previous
+ * call's contents, which the next call overwrites as far as it reads them.  Synchronous, null
+ * stream of the current device. */
+#define MGEMV_STATIC_SCRATCH_BYTES (16u << 20)
+MGEMV_API int mgemv_host_gemv_static(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t *weights,
+                                     const uint16_t *x, const uint16_t *scale, const int8_t *zero_point,
+                                     const uint16_t *bias, uint16_t *y, int quant_op, int weight_bits);
+/* Bytes of the static arrays such a call would use (0 if the arguments are not a legal problem). */
+MGEMV_API size_t mgemv_static_scratch_bytes_needed(int n_out, int m_batch, int k, int group_size, int quant_op,
+                                                   int weight_bits, int has_bias);
 
 /* Parity/debug entry: writes the dequantised weights, fp16 [n_out][k] row-major, produced by
  * the SAME device conversion and dequantisation code the GEMV kernels use

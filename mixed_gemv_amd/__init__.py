@@ -16,6 +16,8 @@ from .api import (  # noqa: F401
     device_gemv,
     gemv_arguments,
     host_gemv,
+    static_scratch_bytes_needed,
+    STATIC_SCRATCH_BYTES,
     probe_empty_launch,
     probe_gemv,
     probe_stream_read,

@@ -185,12 +185,24 @@ def gemv_arguments(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, M, N, 
     _lib.check(_lib.lib().mgemv_gemv_arguments(ctypes.byref(a), _stream_ptr(stream)), "gemv_arguments")
 
 
+STATIC_SCRATCH_BYTES = 16 << 20
+
+
+def static_scratch_bytes_needed(M, N, K, group_size, quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS,
+                                weight_bits=4, has_bias=False):
+    """Bytes of the static arrays host_gemv(..., static_scratch=True) would use; 0 for an illegal problem."""
+    return int(_lib.lib().mgemv_static_scratch_bytes_needed(int(M), int(N), int(K), int(group_size), int(quant_op),
+                                                            int(weight_bits), 1 if has_bias else 0))
+
+
 def host_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, B, M, N, K, group_size,
-              quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4):
+              quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS, weight_bits=4, static_scratch=False):
     """host_gemv of mixed_gemv_test.cu:167-181, i.e. host::reference::MixedGemv::operator()
     (host/mixed_gemv.h:60-70), with the GPU behind it: numpy arrays in host memory, UN-preprocessed
     packed weights [M][K], int8 zero points [K/group_size][M] (mode 3), optional fp16 bias.  Returns
-    the fp16 result [N][M].  There is no CPU path: without a gfx950 device this raises."""
+    the fp16 result [N][M].  There is no CPU path: without a gfx950 device this raises.
+    static_scratch=True calls mgemv_host_gemv_static, which allocates nothing (problems up to
+    STATIC_SCRATCH_BYTES of staging)."""
     w = np.ascontiguousarray(ptr_A).reshape(-1).view(np.uint8)
     x = np.ascontiguousarray(ptr_B, dtype=np.float16)
     s = np.ascontiguousarray(ptr_scale, dtype=np.float16)
@@ -201,10 +213,10 @@ def host_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, B, M, N, K, group_
         raise ValueError("operand smaller than the problem")
     y = np.empty((int(N), int(M)), dtype=np.float16)
     null = ctypes.c_void_p(0)
-    st = _lib.lib().mgemv_host_gemv(int(B), int(M), int(N), int(K), int(group_size), _host_ptr(w), _host_ptr(x),
-                                    _host_ptr(s), _host_ptr(z) if z is not None else null,
-                                    _host_ptr(b) if b is not None else null, _host_ptr(y), int(quant_op),
-                                    int(weight_bits))
+    fn = _lib.lib().mgemv_host_gemv_static if static_scratch else _lib.lib().mgemv_host_gemv
+    st = fn(int(B), int(M), int(N), int(K), int(group_size), _host_ptr(w), _host_ptr(x), _host_ptr(s),
+            _host_ptr(z) if z is not None else null, _host_ptr(b) if b is not None else null, _host_ptr(y),
+            int(quant_op), int(weight_bits))
     _lib.check(st, "host_gemv")
     return y
 

@@ -696,10 +696,18 @@ int mgemv_gemv_arguments(const mgemv_arguments* a, void* stream) {
 }
 
 // host/mixed_gemv.h:60-70 on the GPU: un-preprocessed weights and int8 zero points in host
-// memory in, result in host memory out.
-int mgemv_host_gemv(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t* weights,
-                    const uint16_t* x, const uint16_t* scale, const int8_t* zero_point, const uint16_t* bias,
-                    uint16_t* y, int quant_op, int weight_bits) {
+// memory in, result in host memory out.  Both entry points below share everything but where their
+// staging memory comes from.
+namespace {
+
+struct HostGemvLayout {
+  size_t tiled_bytes, table, off_w, off_x, off_s, off_z, off_b, off_y, total;
+  bool has_zero;
+};
+
+int host_gemv_layout(int batch, int n_out, int m_batch, int k, int& group_size, const void* weights, const void* x,
+                     const void* scale, const void* zero_point, const void* y, bool has_bias, int quant_op, int weight_bits,
+                     HostGemvLayout& l) {
   if (batch != 1) return MGEMV_ERR_BATCH;  // host/mixed_gemv.h:77-80
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
   if (weights == nullptr || x == nullptr || scale == nullptr || y == nullptr) return MGEMV_ERR_NULL_POINTER;
@@ -707,49 +715,133 @@ int mgemv_host_gemv(int batch, int n_out, int m_batch, int k, int group_size, co
       quant_op != MGEMV_FINEGRAINED_SCALE_AND_ZEROS)
     return MGEMV_ERR_QUANT_OP;
   if (weight_bits != 4 && weight_bits != 8) return MGEMV_ERR_QUANT_TYPE;
-  const bool has_zero = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
-  if (has_zero && zero_point == nullptr) return MGEMV_ERR_NULL_POINTER;
+  l.has_zero = quant_op == MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  if (l.has_zero && zero_point == nullptr) return MGEMV_ERR_NULL_POINTER;
   if (n_out <= 0 || k <= 0) return MGEMV_ERR_SIZE;
   if (quant_op == MGEMV_PER_COLUMN_SCALE_ONLY) group_size = k;
   if (group_size <= 0 || k % group_size) return MGEMV_ERR_GROUP_SIZE;
-  const size_t groups = (size_t)(k / group_size), table = groups * (size_t)n_out;
+  if (n_out % 4) return MGEMV_ERR_ROWS;  // what the preprocessor would refuse (utils/preprocess.h:319-327),
+  if (k % 8) return MGEMV_ERR_COLS;      // before any memory is touched
+  l.table = (size_t)(k / group_size) * (size_t)n_out;
+  const size_t shape[2] = {(size_t)k, (size_t)n_out};
+  l.tiled_bytes = mgemv_preprocessed_size(shape, 2, weight_bits == 4 ? MGEMV_W4_A16 : MGEMV_W8_A16);
+  // one piece of memory, 256-byte aligned parts
+  auto align = [](size_t v) { return (v + 255) / 256 * 256; };
+  l.off_w = 0;
+  l.off_x = l.off_w + align(l.tiled_bytes);
+  l.off_s = l.off_x + align((size_t)m_batch * k * 2);
+  l.off_z = l.off_s + align(l.table * 2);
+  l.off_b = l.off_z + align(l.has_zero ? l.table * 2 : 0);
+  l.off_y = l.off_b + align(has_bias ? (size_t)n_out * 2 : 0);
+  l.total = l.off_y + align((size_t)m_batch * n_out * 2);
+  return MGEMV_OK;
+}
 
+// dev: device staging of l.total bytes; host_stage: host memory laid out the same way, of which the
+// weight and zero parts are used.
+int host_gemv_staged(const HostGemvLayout& l, uint8_t* dev, uint8_t* host_stage, int n_out, int m_batch, int k,
+                     int group_size, const uint8_t* weights, const uint16_t* x, const uint16_t* scale,
+                     const int8_t* zero_point, const uint16_t* bias, uint16_t* y, int quant_op, int weight_bits) {
   const size_t shape[2] = {(size_t)k, (size_t)n_out};
   const int quant_type = weight_bits == 4 ? MGEMV_W4_A16 : MGEMV_W8_A16;
-  std::vector<uint8_t> tiled(mgemv_preprocessed_size(shape, 2, quant_type));
-  if (const int st = mgemv_preprocess_weights(tiled.data(), weights, shape, 2, MGEMV_COLUMN_MAJOR, quant_type)) return st;
-  std::vector<uint16_t> zero_add;
-  if (has_zero) {
-    zero_add.resize(table);
-    if (const int st = mgemv_fold_zero_points(zero_add.data(), scale, zero_point, table)) return st;  // utils/preprocess.h:94-101
+  uint8_t* const tiled = host_stage + l.off_w;
+  if (const int st = mgemv_preprocess_weights(tiled, weights, shape, 2, MGEMV_COLUMN_MAJOR, quant_type)) return st;
+  uint16_t* const zero_add = reinterpret_cast<uint16_t*>(host_stage + l.off_z);
+  if (l.has_zero) {
+    if (const int st = mgemv_fold_zero_points(zero_add, scale, zero_point, l.table)) return st;  // utils/preprocess.h:94-101
   }
-
-  // one device allocation, 256-byte aligned pieces
-  auto align = [](size_t v) { return (v + 255) / 256 * 256; };
-  const size_t off_w = 0, off_x = off_w + align(tiled.size()), off_s = off_x + align((size_t)m_batch * k * 2),
-               off_z = off_s + align(table * 2), off_b = off_z + align(has_zero ? table * 2 : 0),
-               off_y = off_b + align(bias ? (size_t)n_out * 2 : 0), total = off_y + align((size_t)m_batch * n_out * 2);
-  uint8_t* dev = nullptr;
-  if (hipMalloc(reinterpret_cast<void**>(&dev), total) != hipSuccess) return MGEMV_ERR_ALLOCATION;
   int st = MGEMV_OK;
   auto up = [&](size_t off, const void* src, size_t bytes) {
     if (st == MGEMV_OK && bytes && hipMemcpy(dev + off, src, bytes, hipMemcpyHostToDevice) != hipSuccess) st = MGEMV_ERR_LAUNCH;
   };
-  up(off_w, tiled.data(), tiled.size());
-  up(off_x, x, (size_t)m_batch * k * 2);
-  up(off_s, scale, table * 2);
-  if (has_zero) up(off_z, zero_add.data(), table * 2);
-  if (bias) up(off_b, bias, (size_t)n_out * 2);
+  up(l.off_w, tiled, l.tiled_bytes);
+  up(l.off_x, x, (size_t)m_batch * k * 2);
+  up(l.off_s, scale, l.table * 2);
+  if (l.has_zero) up(l.off_z, zero_add, l.table * 2);
+  if (bias) up(l.off_b, bias, (size_t)n_out * 2);
   if (st == MGEMV_OK)
-    st = mgemv_gemv(dev + off_w, reinterpret_cast<const uint16_t*>(dev + off_x), reinterpret_cast<const uint16_t*>(dev + off_s),
-                    has_zero ? reinterpret_cast<const uint16_t*>(dev + off_z) : nullptr,
-                    bias ? reinterpret_cast<const uint16_t*>(dev + off_b) : nullptr, reinterpret_cast<uint16_t*>(dev + off_y),
-                    n_out, m_batch, k, group_size, quant_op, weight_bits, nullptr);
+    st = mgemv_gemv(dev + l.off_w, reinterpret_cast<const uint16_t*>(dev + l.off_x),
+                    reinterpret_cast<const uint16_t*>(dev + l.off_s),
+                    l.has_zero ? reinterpret_cast<const uint16_t*>(dev + l.off_z) : nullptr,
+                    bias ? reinterpret_cast<const uint16_t*>(dev + l.off_b) : nullptr,
+                    reinterpret_cast<uint16_t*>(dev + l.off_y), n_out, m_batch, k, group_size, quant_op, weight_bits, nullptr);
   // the blocking copy on the null stream is ordered behind the kernel
-  if (st == MGEMV_OK && hipMemcpy(y, dev + off_y, (size_t)m_batch * n_out * 2, hipMemcpyDeviceToHost) != hipSuccess)
+  if (st == MGEMV_OK && hipMemcpy(y, dev + l.off_y, (size_t)m_batch * n_out * 2, hipMemcpyDeviceToHost) != hipSuccess)
     st = MGEMV_ERR_LAUNCH;
+  return st;
+}
+
+}  // namespace
+
+int mgemv_host_gemv(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t* weights,
+                    const uint16_t* x, const uint16_t* scale, const int8_t* zero_point, const uint16_t* bias,
+                    uint16_t* y, int quant_op, int weight_bits) {
+  HostGemvLayout l{};
+  if (const int st = host_gemv_layout(batch, n_out, m_batch, k, group_size, weights, x, scale, zero_point, y,
+                                      bias != nullptr, quant_op, weight_bits, l))
+    return st;
+  std::vector<uint8_t> host_stage(l.off_b);  // the weight and zero parts are what the host side fills
+  uint8_t* dev = nullptr;
+  if (hipMalloc(reinterpret_cast<void**>(&dev), l.total) != hipSuccess) return MGEMV_ERR_ALLOCATION;
+  const int st = host_gemv_staged(l, dev, host_stage.data(), n_out, m_batch, k, group_size, weights, x, scale, zero_point,
+                                  bias, y, quant_op, weight_bits);
   (void)hipFree(dev);
   return st;
+}
+
+// The allocation-free variant: the same staging in a static device array (one copy per GPU, at
+// its own address there) and a static host array.  The array's name is a host-side handle, not a
+// device address: host code only ever uses the pointer hipGetSymbolAddress returned for the
+// device at hand.
+static __device__ __align__(256) unsigned char scratch[MGEMV_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxScratchDevices = 64;
+alignas(256) unsigned char g_static_host_stage[MGEMV_STATIC_SCRATCH_BYTES];
+unsigned char* g_scratch_of_device[kMaxScratchDevices];  // what hipGetSymbolAddress gave, per device
+std::mutex g_static_mutex;                               // one call at a time: the arrays are shared
+
+// The address of `scratch` on the current device (looked up once per device, with it current).
+int static_scratch_of_current_device(unsigned char*& ptr) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) return MGEMV_ERR_NO_DEVICE;
+  if (device < 0 || device >= kMaxScratchDevices) return MGEMV_ERR_NO_DEVICE;
+  if (g_scratch_of_device[device] == nullptr) {
+    mgemv::DeviceInfo info{};
+    if (const int st = mgemv::device_info(device, info)) return st;  // gfx950 only: other devices hold no copy of the array
+    unsigned char* p = nullptr;
+    if (hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr)
+      return MGEMV_ERR_NO_DEVICE;
+    g_scratch_of_device[device] = p;
+  }
+  ptr = g_scratch_of_device[device];
+  return MGEMV_OK;
+}
+}  // namespace
+
+size_t mgemv_static_scratch_bytes_needed(int n_out, int m_batch, int k, int group_size, int quant_op, int weight_bits,
+                                         int has_bias) {
+  HostGemvLayout l{};
+  static const int dummy = 0;  // the layout only asks whether the pointers are there
+  if (host_gemv_layout(1, n_out, m_batch, k, group_size, &dummy, &dummy, &dummy, &dummy, &dummy, has_bias != 0, quant_op,
+                       weight_bits, l))
+    return 0;
+  return l.total;
+}
+
+int mgemv_host_gemv_static(int batch, int n_out, int m_batch, int k, int group_size, const uint8_t* weights,
+                           const uint16_t* x, const uint16_t* scale, const int8_t* zero_point, const uint16_t* bias,
+                           uint16_t* y, int quant_op, int weight_bits) {
+  HostGemvLayout l{};
+  if (const int st = host_gemv_layout(batch, n_out, m_batch, k, group_size, weights, x, scale, zero_point, y,
+                                      bias != nullptr, quant_op, weight_bits, l))
+    return st;
+  if (l.total > MGEMV_STATIC_SCRATCH_BYTES) return MGEMV_ERR_SCRATCH_SIZE;
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  unsigned char* dev = nullptr;
+  if (const int st = static_scratch_of_current_device(dev)) return st;
+  return host_gemv_staged(l, dev, g_static_host_stage, n_out, m_batch, k, group_size, weights, x, scale, zero_point, bias, y,
+                          quant_op, weight_bits);
 }
 
 int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgroup, int tiles_per_wave, int max_workgroups) {

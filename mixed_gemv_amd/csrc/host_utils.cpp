@@ -293,6 +293,7 @@ const char* mgemv_status_string(int status) {
     case MGEMV_ERR_LAYOUT: return "layout must be 0 (row major) or 1 (column major)";
     case MGEMV_ERR_LEADING_DIMENSION: return "a leading dimension or batch stride describes an operand this library does not take (only the reference's dense operands)";
     case MGEMV_ERR_ALLOCATION: return "device memory could not be allocated (host-pointer entry point)";
+    case MGEMV_ERR_SCRATCH_SIZE: return "the problem does not fit the static scratch arrays of the allocation-free host-pointer entry point";
     case MGEMV_ERR_SIZE: return "a dimension is zero, negative or exceeds the 32-bit index range of the kernels";
     case MGEMV_ERR_LAUNCH: return "HIP launch failed";
     case MGEMV_ERR_NO_DEVICE: return "no usable gfx950 device";
@@ -301,6 +302,6 @@ const char* mgemv_status_string(int status) {
   }
 }
 
-int mgemv_version(void) { return 211; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
+int mgemv_version(void) { return 212; }  // 2xx: int4 fields at bits 7-10 / 3-6 of each half-word
 
 }  // extern "C"

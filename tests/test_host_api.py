@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(handle, name), f"{name} declared in include/mixed_gemv.h but not exported"
     assert declared == set(_lib.SIGNATURES), "python binding and header disagree"
     assert _lib.lib().mgemv_version() >= 100
-    for code in range(0, 16):
+    for code in range(0, 17):
         assert _lib.lib().mgemv_status_string(code) not in (None, b"", b"unknown status")
 
 
@@ -266,7 +266,8 @@ def test_device_entry_points_report_a_missing_device():
     assert lib.mgemv_dequantize(p, p, p, p, 64, 512, 128, 3, 4, None) == 12
 
 
-def test_host_gemv_checks_its_arguments_before_touching_the_device():
+@pytest.mark.parametrize("entry", ["mgemv_host_gemv", "mgemv_host_gemv_static"])
+def test_host_gemv_checks_its_arguments_before_touching_the_device(entry):
     lib = _lib.lib()
     w = np.zeros(64 * 512 // 2, dtype=np.uint8)
     h = np.zeros(64 * 512, dtype=np.uint16)
@@ -274,7 +275,7 @@ def test_host_gemv_checks_its_arguments_before_touching_the_device():
     ptr = lambda a: ctypes.c_void_p(a.ctypes.data)  # noqa: E731
 
     def call(batch=1, n=64, m=1, k=512, g=128, ww=w, x=h, s=h, zz=z, y=h, qop=3, bits=4):
-        return lib.mgemv_host_gemv(batch, n, m, k, g, ptr(ww) if ww is not None else None, ptr(x), ptr(s),
+        return getattr(lib, entry)(batch, n, m, k, g, ptr(ww) if ww is not None else None, ptr(x), ptr(s),
                                    ptr(zz) if zz is not None else None, None, ptr(y), qop, bits)
 
     assert call(batch=2) == 8                      # host/mixed_gemv.h:77-80
@@ -283,6 +284,27 @@ def test_host_gemv_checks_its_arguments_before_touching_the_device():
     assert call(qop=0) == 6 and call(bits=3) == 7
     assert call(g=100) == 5
     assert call(n=66) == 3 and call(k=516, g=516) == 4
+
+
+def test_static_scratch_limit_is_checked_on_the_host():
+    """mgemv_host_gemv_static refuses a problem whose staging exceeds its static arrays before it
+    looks for a device; the size query agrees with the layout both host-pointer entries use."""
+    lib = _lib.lib()
+    limit = mg.STATIC_SCRATCH_BYTES
+    assert limit == 16 << 20
+    # weights + activations + scales + folded zeros + outputs, each piece rounded up to 256 bytes
+    need = mg.static_scratch_bytes_needed(4096, 1, 4096, 128)
+    assert need == 4096 * 4096 // 2 + 4096 * 2 + 2 * (32 * 4096 * 2) + 4096 * 2
+    assert mg.static_scratch_bytes_needed(4096, 1, 4096, 128, has_bias=True) == need + 4096 * 2
+    assert mg.static_scratch_bytes_needed(100, 3, 1120, 160) == (
+        7 * 3 * 4096 + 6912 + 2 * 1536 + 768)   # 7 tiles x 3 k steps; 3 x 1120 x 2 = 6720 -> 6912; 7 x 100 x 2 = 1400 -> 1536; 600 -> 768
+    assert mg.static_scratch_bytes_needed(4096, 1, 4096, 100) == 0 and mg.static_scratch_bytes_needed(4096, 17, 4096, 128) == 0
+    n_out, k = 8192, 8192
+    assert mg.static_scratch_bytes_needed(n_out, 1, k, 128) > limit
+    dummy = np.zeros(16, dtype=np.uint16)   # never read: the size check comes first
+    p = ctypes.c_void_p(dummy.ctypes.data)
+    assert lib.mgemv_host_gemv_static(1, n_out, 1, k, 128, p, p, p, p, None, p, 3, 4) == 16
+    assert b"static scratch" in lib.mgemv_status_string(16)
 
 
 def test_tuned_plan_table_steers_exactly_its_problem(tmp_path):
