@@ -322,6 +322,7 @@ def ceilings_of(wl, use_graph, timeline=False):
                     shape of the GEMV and for the best of a few others (no scales, no activations,
                     no arithmetic): us per launch and GB/s of the bytes read;
       loads_only    the GEMV kernel itself with every load kept and the arithmetic removed;
+      compute_only  the GEMV kernel itself with the arithmetic kept and only each wave's first unit loaded;
       timeline      (headline only) when the phases of one launch happen."""
     import statistics
     import torch
@@ -354,6 +355,13 @@ def ceilings_of(wl, use_graph, timeline=False):
     out["loads_only"] = {"us_per_launch": round(ev_us, 3), "GBps": round(wl.bytes / ev_us / 1e3, 1),
                          "frac_of_hbm_peak": round(wl.bytes / ev_us / 1e3 / HBM_PEAK_GBS, 4),
                          "note": "the GEMV kernel with its weight, activation, scale and zero loads and no arithmetic"}
+    probe = _Launches(lambda i: mg.probe_gemv(mg.PROBE_COMPUTE_ONLY, None, wl.w[i % wl.sets], wl.x, wl.s[i % wl.sets],
+                                              wl.z[i % wl.sets], wl.y, wl.n_out, wl.k, wl.group), wl.sets)
+    _, ev_us, *_ = time_workload(probe, 400, 20, use_graph=use_graph, repetitions=5)
+    units_per_wave = plan["steps_per_wave"] * plan["tiles_in_sequence"]
+    out["compute_only"] = {"us_per_launch": round(ev_us, 3), "units_per_wave": units_per_wave,
+                           "note": "the GEMV kernel with its arithmetic kept (dequantise + dot of every unit, combine, store) "
+                                   "and only the first unit of each wave loaded"}
     if timeline:
         n_waves = plan["workgroups"] * waves
         trace = torch.zeros((n_waves, 5), dtype=torch.int64, device=wl.y.device)

@@ -403,8 +403,11 @@ MGEMV_API int mgemv_probe_stream_read(const void *src, size_t bytes, int workgro
  *                           and threads as mgemv_query_launch reports): i = 0 the wave starts,
  *                           1 its first unit is requested, 2 that unit's first block has arrived,
  *                           3 its last unit is computed, 4 its outputs are stored.  y is the
- *                           GEMV's result. */
-enum { MGEMV_PROBE_LOADS_ONLY = 1, MGEMV_PROBE_TIMELINE = 2 };
+ *                           GEMV's result;
+ *   MGEMV_PROBE_COMPUTE_ONLY every wave loads the first unit of its range and then runs the
+ *                           arithmetic of that unit once per unit of the range, loading nothing
+ *                           more: what the kernel's instructions alone take; y is meaningless. */
+enum { MGEMV_PROBE_LOADS_ONLY = 1, MGEMV_PROBE_TIMELINE = 2, MGEMV_PROBE_COMPUTE_ONLY = 3 };
 MGEMV_API int mgemv_probe_gemv(int kind, unsigned long long *trace, const void *weights, const uint16_t *x,
                                const uint16_t *scale, const uint16_t *zero_add, uint16_t *y, int n_out, int k,
                                int group_size, void *stream);

@@ -362,6 +362,7 @@ def set_prefetch_stages(stages):
 
 PROBE_LOADS_ONLY = 1
 PROBE_TIMELINE = 2
+PROBE_COMPUTE_ONLY = 3
 
 
 def probe_empty_launch(stream=None):
@@ -377,7 +378,7 @@ def probe_stream_read(src, nbytes, workgroups, waves_per_workgroup, units_in_fli
 
 
 def probe_gemv(kind, trace, ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_D, M, K, group_size, stream=None):
-    """Measurement builds of the headline kernel (mgemv_probe_gemv): PROBE_LOADS_ONLY or PROBE_TIMELINE
+    """Measurement builds of the headline kernel (mgemv_probe_gemv): PROBE_LOADS_ONLY, PROBE_COMPUTE_ONLY or PROBE_TIMELINE
     (trace: int64 device tensor of 5 entries per wave)."""
     _lib.check(_lib.lib().mgemv_probe_gemv(int(kind), _dev_ptr(trace), _dev_ptr(ptr_A), _dev_ptr(ptr_B),
                                            _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_D), int(M), int(K),

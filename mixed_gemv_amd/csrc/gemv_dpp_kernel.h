@@ -168,6 +168,21 @@ __device__ __forceinline__ void load_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>
   load_weights<BITS, MB, GROUPS_PER_RUN>(f, w_rsrc, c.w_voffset);
 }
 
+// Measurement build "arithmetic only": a wave loads its first unit and computes that unit's
+// registers again for every further unit of its range.  Nothing is loaded; the registers are made
+// opaque each time so that no part of the arithmetic can be hoisted out of the unit loop.
+template <int BITS, int MB, int GROUPS_PER_RUN>
+__device__ __forceinline__ void reuse_unit(UnitFragment<BITS, MB, GROUPS_PER_RUN>& f) {
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) asm volatile("" : "+v"(f.w[i]));
+#pragma unroll
+  for (int m = 0; m < MB; ++m)
+#pragma unroll
+    for (int h = 0; h < (BITS == 4 ? 4 : 2); ++h) asm volatile("" : "+v"(f.x[m][h]));
+#pragma unroll
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) asm volatile("" : "+v"(f.s[gi]), "+v"(f.z[gi]));
+}
+
 // One 32-bit word of block I: convert, dequantise, dot.  Lane (4 I + J) of the DPP row holds
 // the activations that pair with this word.  SHORT selects the single-FMA int4 dequantiser
 // (device_math.h); the caller guarantees that every lane's scale permits it.
@@ -311,7 +326,8 @@ __device__ __forceinline__ void finish_tile(float (&acc)[MB], float* slot) {
 // ACT: kActF16 or kActBf16 -- the type of activations, scales, zeros, bias and outputs (the
 // pointers are typed as 16-bit storage either way).
 // PROBE (measurement builds of this same kernel, see mixed_gemv.h "Measurement probes"):
-// kProbeNone the product; kProbeLoadsOnly keeps every load and replaces the arithmetic of a unit
+// kProbeNone the product; kProbeComputeOnly loads a wave's first unit only and repeats its arithmetic
+// for every further unit; kProbeLoadsOnly keeps every load and replaces the arithmetic of a unit
 // by an exclusive-or over its registers -- what the access pattern alone takes; kProbeTimeline
 // records five timestamps per wave.
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI, int ACT, int PROBE = kProbeNone>
@@ -403,6 +419,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       stamp[2] = __builtin_amdgcn_s_memrealtime();
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (PROBE == kProbeComputeOnly) fb = fa;  // (waits for the first unit; every later "load" re-uses it)
     const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
     const ConvertRegs c = make_convert_regs();
     // With two or more activation rows, a wave of exactly two units runs straight-line code: the
@@ -416,7 +433,8 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       if constexpr (MULTI) finish_tile<MB>(acc, slot);
     } else if (MB >= 2 && !MULTI && total == 2) {
       advance<MULTI>(cur, walk);
-      load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
+      if constexpr (PROBE == kProbeComputeOnly) reuse_unit<BITS, MB, GROUPS_PER_RUN>(fb);
+      else load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
       __builtin_amdgcn_sched_barrier(0);
       compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
       __builtin_amdgcn_sched_barrier(0);
@@ -434,7 +452,8 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       int u = 0;
       do {
         advance<MULTI>(cur, walk);
-        load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
+        if constexpr (PROBE == kProbeComputeOnly) reuse_unit<BITS, MB, GROUPS_PER_RUN>(fb);
+        else load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
         if (single_stage) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
         compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
@@ -446,7 +465,8 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         }
         advance<MULTI>(cur, walk);
         __builtin_amdgcn_sched_barrier(0);
-        load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
+        if constexpr (PROBE == kProbeComputeOnly) reuse_unit<BITS, MB, GROUPS_PER_RUN>(fa);
+        else load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
         if (single_stage) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         if (u + 1 < total) {

@@ -669,11 +669,14 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
 
 int mgemv_probe_gemv(int kind, unsigned long long* trace, const void* weights, const uint16_t* x, const uint16_t* scale,
                      const uint16_t* zero_add, uint16_t* y, int n_out, int k, int group_size, void* stream) {
-  if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_TIMELINE) return MGEMV_ERR_SIZE;
+  if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_TIMELINE && kind != MGEMV_PROBE_COMPUTE_ONLY) return MGEMV_ERR_SIZE;
   if (kind == MGEMV_PROBE_TIMELINE && (trace == nullptr || reinterpret_cast<uintptr_t>(trace) % 8)) return MGEMV_ERR_NULL_POINTER;
   return mgemv::gemv_any(weights, x, scale, zero_add, nullptr, y, 1, n_out, 1, k, group_size,
                          MGEMV_FINEGRAINED_SCALE_AND_ZEROS, 4, 0, 0, 0, 0, 0, stream, mgemv::kActF16, 1.0f, 1.0f,
-                         kind == MGEMV_PROBE_LOADS_ONLY ? mgemv::kProbeLoadsOnly : mgemv::kProbeTimeline, trace);
+                         kind == MGEMV_PROBE_LOADS_ONLY     ? mgemv::kProbeLoadsOnly
+                         : kind == MGEMV_PROBE_COMPUTE_ONLY ? mgemv::kProbeComputeOnly
+                                                            : mgemv::kProbeTimeline,
+                         trace);
 }
 
 // gemv/device/gemv_adaptor.h:114-178 as one plain struct.

@@ -20,7 +20,7 @@ constexpr int kNumCus = 256;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
 constexpr int kSingleStage = 2;           // GemvTail::flags: no load in flight while a unit is computed (VALU kernel)
-constexpr int kProbeNone = 0, kProbeLoadsOnly = 1, kProbeTimeline = 2;  // measurement builds of the VALU kernel
+constexpr int kProbeNone = 0, kProbeLoadsOnly = 1, kProbeTimeline = 2, kProbeComputeOnly = 3;  // measurement builds of the VALU kernel
 
 // Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are what a
 // wave needs to address its first loads, and they are preloaded into SGPRs (build flag
@@ -235,7 +235,7 @@ hipError_t launch_gemv_f16(const GemvLaunch& g, int bits, int qop, int mb, int g
 hipError_t launch_gemv_bf16(const GemvLaunch& g, int bits, int qop, int mb, int gpr);
 hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr);
 hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act);
-// Measurement builds of the single-row int4 scale-and-zero fp16 VALU kernel (probe: kProbeLoadsOnly / kProbeTimeline).
+// Measurement builds of the single-row int4 scale-and-zero fp16 VALU kernel (probe: kProbeLoadsOnly / kProbeTimeline / kProbeComputeOnly).
 hipError_t launch_gemv_probe(const GemvLaunch& g, int probe);
 
 }  // namespace mgemv

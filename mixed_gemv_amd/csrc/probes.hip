@@ -1,7 +1,7 @@
 // Measurement probes: the kernels behind the "ceilings" that the benchmark reports beside the
 // GEMV figures -- what an empty launch costs, what a plain streaming read of the same bytes with
-// the same launch shape achieves, what the GEMV's own loads take with the arithmetic removed,
-// and when the phases of one launch happen.  None of this is on a product path and nothing here
+// the same launch shape achieves, what the GEMV's own loads take with the arithmetic removed and
+// its arithmetic with the loads removed, and when the phases of one launch happen.  None of this is on a product path and nothing here
 // has a counterpart in the reference.
 #include "gemv_dpp_kernel.h"
 
@@ -61,7 +61,11 @@ hipError_t launch_gemv_probe_kind(const GemvLaunch& g) {
 }
 
 hipError_t launch_gemv_probe(const GemvLaunch& g, int probe) {
-  return probe == kProbeLoadsOnly ? launch_gemv_probe_kind<kProbeLoadsOnly>(g) : launch_gemv_probe_kind<kProbeTimeline>(g);
+  switch (probe) {
+    case kProbeLoadsOnly: return launch_gemv_probe_kind<kProbeLoadsOnly>(g);
+    case kProbeComputeOnly: return launch_gemv_probe_kind<kProbeComputeOnly>(g);
+    default: return launch_gemv_probe_kind<kProbeTimeline>(g);
+  }
 }
 
 }  // namespace mgemv

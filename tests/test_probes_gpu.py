@@ -36,6 +36,30 @@ def test_timeline_build_is_the_product_kernel_plus_timestamps(gpu, n_out, k, cap
         mg.set_launch_override(0, 0, 0, 0)
 
 
+@pytest.mark.parametrize("n_out,k,split", [(640, 512, 0), (320, 2048, 4), (4096, 4096, 0)])
+def test_compute_only_build_repeats_the_first_unit(gpu, n_out, k, split):
+    """With one unit per wave (one k step, or as many k-split waves as k steps) the arithmetic-only
+    build loads everything the product loads: same bits.  With more units per wave it runs and
+    writes finite-or-not garbage that must simply not fault."""
+    import torch
+    prob = Problem("probe_c", n_out, k, 4, SCALE_AND_ZEROS, 128, x_dist="normal")
+    dev = DeviceProblem(prob, gpu)
+    try:
+        mg.set_launch_override(split, 0, 0, 0)
+        plan = mg.query_launch(n_out, 1, k, 4, 128)
+        want = dev.run().copy()
+        dev.y.fill_(0x7e00)
+        mg.probe_gemv(mg.PROBE_COMPUTE_ONLY, None, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 128)
+        torch.cuda.synchronize()
+        got = dev.y.cpu().numpy().view(np.uint16)
+        if plan["steps_per_wave"] * plan["tiles_in_sequence"] == 1:
+            assert np.array_equal(got.reshape(-1), want.view(np.uint16).reshape(-1))
+        else:
+            assert not np.any(got == 0x7e00)    # every output was written
+    finally:
+        mg.set_launch_override(0, 0, 0, 0)
+
+
 def test_stream_read_and_empty_launch_run_and_check_their_arguments(gpu):
     import torch
     buf = torch.zeros(8 << 20, dtype=torch.uint8, device=gpu)
