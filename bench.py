@@ -665,6 +665,9 @@ def main():
         out["other_workloads"] = others
         out["all_parity_ok"] = bool(out.get("parity", {}).get("ok", True)
                                     and all(e.get("parity", {}).get("ok", True) for e in others.values()))
+    out["launch_plans"] = {"built_in_table_entries": mg.default_plan_count(), "caller_table_entries": mg.tuned_plan_count(),
+                           "note": "rules of plan_launch plus the library's compiled-in table (mixed_gemv_amd/default_plans.json); "
+                                   "nothing is tuned or installed by this run"}
     print(json.dumps(out))
 
 

@@ -339,6 +339,14 @@ MGEMV_API int mgemv_tuned_plan_set(const mgemv_tuned_plan *plan);
 /* Removes the entry with exactly plan's key fields, if there is one (the other fields are not read). */
 MGEMV_API int mgemv_tuned_plan_erase(const mgemv_tuned_plan *plan);
 MGEMV_API int mgemv_tuned_plan_clear(void);
+/* The library also carries a built-in table of the same kind (mixed_gemv_amd/default_plans.json,
+ * compiled in): plans measured on an unpartitioned MI355X that the built-in rules do not produce.
+ * It is consulted after the caller's table, for launches on a device of 256 compute units only, and
+ * bypassed like the caller's table while a process-wide override is set.
+ * mgemv_set_default_plans(0) switches it off (1 on again); mgemv_default_plan_count tells how many
+ * entries it has. */
+MGEMV_API int mgemv_set_default_plans(int enable);
+MGEMV_API int mgemv_default_plan_count(void);
 MGEMV_API int mgemv_tuned_plan_count(void);
 
 /* Reports the geometry mgemv_gemv would use for this problem (group_size as passed to mgemv_gemv,

@@ -41,6 +41,8 @@ from .api import (  # noqa: F401
     erase_tuned_plan,
     set_tuned_plan,
     clear_tuned_plans,
+    default_plan_count,
+    set_default_plans,
     tuned_plan_count,
     KERNEL_AUTO,
     KERNEL_VALU,

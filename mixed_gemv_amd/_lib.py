@@ -52,6 +52,8 @@ SIGNATURES = {
     "mgemv_tuned_plan_set": (_c.c_int, [_c.POINTER(_c.c_int * 12)]),
     "mgemv_tuned_plan_erase": (_c.c_int, [_c.POINTER(_c.c_int * 12)]),
     "mgemv_tuned_plan_clear": (_c.c_int, []),
+    "mgemv_set_default_plans": (_c.c_int, [_c.c_int]),
+    "mgemv_default_plan_count": (_c.c_int, []),
     "mgemv_tuned_plan_count": (_c.c_int, []),
 }
 

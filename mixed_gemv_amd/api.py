@@ -408,6 +408,15 @@ def erase_tuned_plan(n_out, k, weight_bits, group_size, m_batch, element="f16"):
     _lib.check(_lib.lib().mgemv_tuned_plan_erase(ctypes.byref(plan)), "erase_tuned_plan")
 
 
+def set_default_plans(enable=True):
+    """Switches the library's built-in tuned-plan table (default_plans.json) on or off."""
+    _lib.check(_lib.lib().mgemv_set_default_plans(1 if enable else 0), "set_default_plans")
+
+
+def default_plan_count():
+    return int(_lib.lib().mgemv_default_plan_count())
+
+
 def clear_tuned_plans():
     _lib.check(_lib.lib().mgemv_tuned_plan_clear(), "clear_tuned_plans")
 

@@ -56,14 +56,43 @@ def lint_device_code(verbose=True):
     return reports
 
 
+DEFAULT_PLANS = os.path.join(PKG_DIR, "default_plans.json")
+KERNEL_IDS = {"auto": 0, "valu": 1, "matrix_core_register_operand": 2, "matrix_core_lds_staged": 3}
+
+
+def write_default_plans(path):
+    """default_plans.json -> the initialiser list of the library's built-in tuned-plan table
+    (one mgemv_tuned_plan per line), included by csrc/gemv_kernels.hip."""
+    import json
+    with open(DEFAULT_PLANS) as f:
+        table = json.load(f)
+    if table.get("format") != 1:
+        raise RuntimeError(f"{DEFAULT_PLANS}: not a tuned-plan table")
+    lines = []
+    for e in table["plans"]:
+        kernel = e.get("kernel", 0)
+        kernel = KERNEL_IDS[kernel] if isinstance(kernel, str) else int(kernel)
+        element = 1 if e.get("element", "f16") == "bf16" else 0
+        fields = [e["n_out"], e["k"], e["weight_bits"], e["group_size"], e["m_batch"], kernel, e.get("split_k", 0),
+                  e.get("tiles_per_wg", 0), e.get("tiles_per_wave", 0), e.get("max_workgroups", 0), e.get("stages", 0),
+                  element]
+        lines.append("{" + ", ".join(str(int(v)) for v in fields) + "},")
+    text = "// generated from mixed_gemv_amd/default_plans.json by mixed_gemv_amd/build.py\n" + "\n".join(lines) + "\n"
+    if not os.path.exists(path) or open(path).read() != text:
+        with open(path, "w") as f:
+            f.write(text)
+    return len(lines)
+
+
 def build_library(verbose=True, extra_flags=(), jobs=None, lint=True):
     os.makedirs(OBJ_DIR, exist_ok=True)
+    write_default_plans(os.path.join(OBJ_DIR, "default_plans.inc"))
     jobs = jobs or min(len(SOURCES), os.cpu_count() or 1, 16)
 
     def compile_one(src):
         obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
         cmd = [hipcc(), *HIP_FLAGS, *extra_flags, "-save-temps=obj", "-I", os.path.join(REPO_DIR, "include"), "-I", CSRC,
-               "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
+               "-I", OBJ_DIR, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.run(cmd, check=True)

@@ -138,9 +138,49 @@ std::mutex g_tuned_mutex;
 std::map<PlanKey, PlanKnobs> g_tuned_plans;
 std::atomic<int> g_tuned_count{0};  // lets the launch path skip the lock while the table is empty
 
-// Process-wide overrides win over the table (they are what a tuner sweeps); then an entry for
-// exactly this group size, then one for any group size, then the built-in rules.
-PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch, int act) {
+// Built-in table: plans measured on an unpartitioned MI355X that the rules below do not produce,
+// kept as data (mixed_gemv_amd/default_plans.json, compiled in by the build) instead of as one
+// more shape threshold in plan_launch.  Consulted after the caller's table, for launches on a
+// device of kDefaultPlanCus compute units only.
+const mgemv_tuned_plan kDefaultPlans[] = {
+#include "default_plans.inc"
+    {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}  // terminator (n_out = 0)
+};
+constexpr int kDefaultPlanCus = 256;
+std::atomic<int> g_default_plans_enabled{1};
+
+int default_plan_count() {
+  int n = 0;
+  while (kDefaultPlans[n].n_out != 0) ++n;
+  return n;
+}
+
+PlanKnobs knobs_of_plan(const mgemv_tuned_plan& plan) {
+  PlanKnobs kn;
+  kn.split_k = plan.split_k_waves;
+  kn.tiles_per_wg = plan.tiles_per_workgroup;
+  kn.tiles_per_wave = plan.tiles_per_wave;
+  kn.workgroups = plan.max_workgroups;
+  kn.stages = plan.stages;
+  switch (plan.kernel) {
+    case MGEMV_KERNEL_VALU: kn.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1; break;
+    case MGEMV_KERNEL_MATRIX_CORE_REGISTER_OPERAND:
+      kn.matrix_core_min_batch = 1;
+      kn.matrix_core_variant = MGEMV_MATRIX_CORE_REGISTER_OPERAND;
+      break;
+    case MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED:
+      kn.matrix_core_min_batch = 1;
+      kn.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
+      break;
+    default: break;
+  }
+  return kn;
+}
+
+// Process-wide overrides win over the tables (they are what a tuner sweeps); then the caller's
+// entry for exactly this group size, then its entry for any group size, then the built-in table,
+// then the built-in rules.
+PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch, int act, int num_cus) {
   PlanKnobs kn;
   kn.split_k = g_override_split_k.load();
   kn.tiles_per_wg = g_override_tiles_per_wg.load();
@@ -151,12 +191,21 @@ PlanKnobs knobs_for(int n_out, int k, int bits, int group_size, int m_batch, int
   kn.stages = g_override_stages.load();
   const bool overridden = kn.split_k || kn.tiles_per_wg || kn.tiles_per_wave || kn.workgroups || kn.stages ||
                           kn.matrix_core_min_batch || kn.matrix_core_variant != MGEMV_MATRIX_CORE_AUTO;
-  if (overridden || g_tuned_count.load() == 0) return kn;
-  std::lock_guard<std::mutex> lock(g_tuned_mutex);
+  if (overridden) return kn;
   const int element = act == kActBf16 ? MGEMV_ELEMENT_BF16 : MGEMV_ELEMENT_F16;
-  auto it = g_tuned_plans.find(PlanKey{n_out, k, bits, group_size, m_batch, element});
-  if (it == g_tuned_plans.end() && group_size != 0) it = g_tuned_plans.find(PlanKey{n_out, k, bits, 0, m_batch, element});
-  return it == g_tuned_plans.end() ? kn : it->second;
+  if (g_tuned_count.load() != 0) {
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    auto it = g_tuned_plans.find(PlanKey{n_out, k, bits, group_size, m_batch, element});
+    if (it == g_tuned_plans.end() && group_size != 0) it = g_tuned_plans.find(PlanKey{n_out, k, bits, 0, m_batch, element});
+    if (it != g_tuned_plans.end()) return it->second;
+  }
+  if (num_cus == kDefaultPlanCus && g_default_plans_enabled.load() != 0) {
+    for (const mgemv_tuned_plan* p = kDefaultPlans; p->n_out != 0; ++p)
+      if (p->n_out == n_out && p->k == k && p->weight_bits == bits && p->m_batch == m_batch && p->element == element &&
+          (p->group_size == group_size || p->group_size == 0))
+        return knobs_of_plan(*p);
+  }
+  return kn;
 }
 
 // Which row counts go to the matrix cores.  From 5 rows the VALU kernel would need a second pass
@@ -495,7 +544,7 @@ int device_info(int device, DeviceInfo& info) {
 
 // The knobs of a problem with the element type taken into account.
 PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_batch, int act, int num_cus = kNumCus) {
-  PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch, act);
+  PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch, act, num_cus);
   knobs.num_cus = num_cus;
   if (act == kActBf16) {
     // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
@@ -902,25 +951,8 @@ int mgemv_tuned_plan_set(const mgemv_tuned_plan* plan) {
   if (plan->element != MGEMV_ELEMENT_F16 && plan->element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
   const int t = plan->tiles_per_wave;
   if (t != 0 && t != 1 && t != 2 && t != 4) return MGEMV_ERR_SIZE;
-  mgemv::PlanKnobs kn;
-  kn.split_k = plan->split_k_waves;
-  kn.tiles_per_wg = plan->tiles_per_workgroup;
-  kn.tiles_per_wave = t;
-  kn.workgroups = plan->max_workgroups;
-  kn.stages = plan->stages;
-  switch (plan->kernel) {
-    case MGEMV_KERNEL_AUTO: break;
-    case MGEMV_KERNEL_VALU: kn.matrix_core_min_batch = MGEMV_MAX_M_BATCH + 1; break;
-    case MGEMV_KERNEL_MATRIX_CORE_REGISTER_OPERAND:
-      kn.matrix_core_min_batch = 1;
-      kn.matrix_core_variant = MGEMV_MATRIX_CORE_REGISTER_OPERAND;
-      break;
-    case MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED:
-      kn.matrix_core_min_batch = 1;
-      kn.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
-      break;
-    default: return MGEMV_ERR_SIZE;
-  }
+  if (plan->kernel < MGEMV_KERNEL_AUTO || plan->kernel > MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED) return MGEMV_ERR_SIZE;
+  const mgemv::PlanKnobs kn = mgemv::knobs_of_plan(*plan);
   std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);
   mgemv::g_tuned_plans[mgemv::PlanKey{plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch,
                                       plan->element}] = kn;
@@ -936,6 +968,13 @@ int mgemv_tuned_plan_erase(const mgemv_tuned_plan* plan) {
   mgemv::g_tuned_count.store((int)mgemv::g_tuned_plans.size());
   return MGEMV_OK;
 }
+
+int mgemv_set_default_plans(int enable) {
+  mgemv::g_default_plans_enabled.store(enable != 0 ? 1 : 0);
+  return MGEMV_OK;
+}
+
+int mgemv_default_plan_count(void) { return mgemv::default_plan_count(); }
 
 int mgemv_tuned_plan_clear(void) {
   std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);

@@ -463,7 +463,11 @@ BUILTIN_PLANS = [
 @pytest.mark.parametrize("shape,want", BUILTIN_PLANS, ids=[f"{s[0]}x{s[2]}_m{s[1]}" for s, _ in BUILTIN_PLANS])
 def test_builtin_launch_rules_on_the_shapes_they_were_measured_on(shape, want):
     n_out, m_batch, k = shape
-    got = mg.query_launch(n_out, m_batch, k, 4, 128)
+    mg.set_default_plans(False)   # the rules themselves, without the built-in table of measured exceptions
+    try:
+        got = mg.query_launch(n_out, m_batch, k, 4, 128)
+    finally:
+        mg.set_default_plans(True)
     assert {key: got[key] for key in want} == want, got
     # every plan covers every tile and every k step, within the workgroup size the kernels allow
     tiles, ksteps = -(-n_out // 16), -(-k // 512)
@@ -495,3 +499,53 @@ def test_int8_weights_keep_two_to_four_rows_on_the_valu_kernel():
     assert [q(8192, m, 8192) for m in (2, 3, 4, 5)] == [0, 0, 0, 2]
     assert [q(4096, m, 11008) for m in (3, 4, 5)] == [0, 0, 2]
     assert [q(28672, m, 8192) for m in (2, 3, 4)] == [0, 2, 2]
+
+
+def test_default_plan_table_is_the_shipped_json_and_applies_to_256_compute_units_only():
+    import json
+    import os
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "..", "default_plans.json")
+    with open(path) as f:
+        table = json.load(f)
+    assert table["format"] == 1 and mg.default_plan_count() == len(table["plans"]) >= 1
+    kinds = {0: 0, 1: 0, 2: 1, 3: 2}   # MGEMV_KERNEL_* -> what query_launch reports as matrix_core
+    for e in table["plans"]:
+        key = (e["n_out"], e["m_batch"], e["k"], e["weight_bits"], e["group_size"])
+        got = mg.query_launch(*key, element=e["element"], num_compute_units=256)
+        mg.set_default_plans(False)
+        try:
+            rules = mg.query_launch(*key, element=e["element"], num_compute_units=256)
+        finally:
+            mg.set_default_plans(True)
+        assert got != rules, "an entry that changes nothing has no business in the table"
+        if e.get("split_k"):
+            assert got["split_k"] == e["split_k"]
+        if e.get("tiles_per_wg"):
+            assert got["tiles_per_wg"] == e["tiles_per_wg"]
+        if e.get("max_workgroups"):
+            assert got["workgroups"] <= -(-e["max_workgroups"] // 8) * 8
+        if e.get("kernel"):
+            assert got["matrix_core"] == kinds[e["kernel"]]
+        assert e["us"] < e["builtin_us"] * 0.98
+        # the entry covers the problem like any plan
+        cov = mg.plan_coverage(*key, element=e["element"], num_compute_units=256)
+        assert cov["tiles_miscovered"] == 0 and cov["bad_waves"] == 0
+        # other device sizes, the other element type, a caller's table entry and any override: not this entry
+        assert mg.query_launch(*key, element=e["element"], num_compute_units=128) == \
+            _with_defaults_off(lambda: mg.query_launch(*key, element=e["element"], num_compute_units=128))
+        other = "bf16" if e["element"] == "f16" else "f16"
+        assert mg.query_launch(*key, element=other, num_compute_units=256) == \
+            _with_defaults_off(lambda: mg.query_launch(*key, element=other, num_compute_units=256))
+        mg.set_prefetch_stages(2)
+        try:
+            assert {k: v for k, v in mg.query_launch(*key, element=e["element"], num_compute_units=256).items()} == rules
+        finally:
+            mg.set_prefetch_stages(0)
+
+
+def _with_defaults_off(fn):
+    mg.set_default_plans(False)
+    try:
+        return fn()
+    finally:
+        mg.set_default_plans(True)
