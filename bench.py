@@ -52,7 +52,7 @@ WORKLOADS = {
 # averaged over the launches of `bench.py --workload <name> --launch stream`), scaled by what the same
 # counters read for a plain 512 MiB device copy on the same box: FETCH_SIZE reads 262155.5 for 524288 KiB
 # (factor 2.0), WRITE_SIZE reads 524288 (factor 1.0).  See profiles/.  name -> (fetch KiB raw, write KiB raw)
-MEASURED_TRAFFIC_KIB = {"ns": (4472.0, 8.0), "c5": (61089.5, 56.0)}
+MEASURED_TRAFFIC_KIB = {"ns": (4466.5, 8.0), "c5": (61110.0, 56.0)}
 FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
 
 
