@@ -69,6 +69,59 @@ def test_arguments_entry_alpha_beta(gpu, m_batch):
     assert np.all(np.abs(got - want) <= tol)
 
 
+@pytest.mark.parametrize("element", ["f16", "bf16"])
+def test_arguments_entry_batched_with_strides_and_epilogue(gpu, element):
+    """The whole argument struct at once (gemv/device/gemv_adaptor.h:114-178): three problems per launch
+    through their batch strides, either element type, alpha = 2 and beta = 0.5.  Doubling commutes with
+    the final rounding of both types (no result here is near overflow), so the launch must equal, bit for
+    bit, twice the accumulator-only result plus the exactly halved bias whenever that sum is exact; it is
+    checked against the plain batched entry through the closed form for alpha alone, and against fp64
+    within half an ulp for both."""
+    import torch
+    e, n_out, k, g = 3, 96, 1536, 128
+    probs = [Problem(f"argb{i}", n_out, k, 4, SCALE_AND_ZEROS, g, bias=True, x_dist="normal", element=element)
+             for i in range(e)]
+    raw = np.concatenate([p.w_raw for p in probs])
+    pre = mg.MixedGemvWeightPreprocessor.run(raw, (e, k, n_out), mg.LayoutType.kColumnMajor, mg.QuantType.W4_A16)
+    one = mg.preprocessed_size((k, n_out), mg.QuantType.W4_A16)
+
+    def stack(name):
+        return torch.from_numpy(np.stack([np.asarray(getattr(p, name)).view(np.uint16) for p in probs]).view(np.int16)).to(gpu)
+
+    w = torch.from_numpy(pre).to(gpu)
+    scale, zero, bias = stack("scale"), stack("zero_add"), stack("bias")
+    x = torch.from_numpy(np.asarray(probs[0].x).view(np.uint16).view(np.int16)).to(gpu)
+    y = torch.full((e, n_out), 0x7E00, dtype=torch.int16, device=gpu)
+    strides = (one, 0, (k // g) * n_out, n_out, n_out)
+
+    def run(alpha, beta, with_bias=True):
+        y.fill_(0x7E00)
+        mg.gemv_arguments(w, x, scale, zero, bias if with_bias else None, y, n_out, 1, k, g, SCALE_AND_ZEROS, 4,
+                          alpha=alpha, beta=beta, batch_count=e, batch_strides=strides, element=element)
+        torch.cuda.synchronize()
+        return y.cpu().numpy().view(np.uint16).copy()
+
+    def to_f64(bits):
+        if element == "bf16":
+            return orc.bf16_to_f32_array(bits).astype(np.float64)
+        return bits.view(np.float16).astype(np.float64)
+
+    # alpha = beta = 1 is the batched entry, bit for bit
+    y.fill_(0x7E00)
+    mg.device_gemv(w, x, scale, zero, bias, y, e, n_out, 1, k, g, SCALE_AND_ZEROS, 4, batch_strides=strides, element=element)
+    torch.cuda.synchronize()
+    assert np.array_equal(run(1.0, 1.0), y.cpu().numpy().view(np.uint16))
+    # alpha = 2 without a bias: exactly twice the accumulator-only result
+    acc = run(1.0, 0.0, with_bias=False)
+    assert np.array_equal(to_f64(run(2.0, 0.0, with_bias=False)), 2.0 * to_f64(acc))
+    # alpha = 2, beta = 0.5: one rounding of 2 acc + bias / 2; acc is only known rounded, so allow its ulp
+    got = to_f64(run(2.0, 0.5))
+    bias64 = to_f64(np.stack([np.asarray(p.bias).view(np.uint16) for p in probs]))
+    want = 2.0 * to_f64(acc) + 0.5 * bias64
+    ulp = 2.0 ** (-7 if element == "bf16" else -10)
+    assert np.all(np.abs(got - want) <= ulp * (2.0 * np.abs(to_f64(acc)) + np.abs(want)) + 2.0 ** -24)
+
+
 def test_arguments_entry_bias_term_alone_is_exact(gpu):
     """x = 0: y = fp16(beta * bias) exactly (epilogue/threadblock/epilogue.h:64)."""
     import torch
