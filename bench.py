@@ -334,6 +334,10 @@ def ceilings_of(wl, use_graph, timeline=False):
     sink = torch.zeros(1, dtype=torch.int32, device=wl.y.device)
     out = {"weight_bytes": w_bytes, "algorithmic_bytes": wl.bytes, "stream_read": []}
     waves = plan["threads"] // 64
+    probe = _Launches(lambda i: mg.probe_empty_grid(plan["workgroups"], waves), 1)
+    _, ev_us, *_ = time_workload(probe, 2000, 100, use_graph=use_graph, repetitions=7)
+    out["empty_grid"] = {"workgroups": plan["workgroups"], "waves_per_workgroup": waves, "us_per_launch": round(ev_us, 3),
+                         "note": "an empty kernel with the GEMV's grid: launch cadence plus the dispatch of its waves"}
     shapes = [("the GEMV's launch shape", plan["workgroups"], waves, 2)]
     shapes += [("", 128, 8, 2), ("", 256, 8, 2), ("", 512, 4, 4), ("", 1024, 4, 4), ("", 512, 8, 8)]
     for label, wgs, wv, depth in shapes:

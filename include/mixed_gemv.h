@@ -392,6 +392,9 @@ MGEMV_API int mgemv_plan_coverage(int n_out, int m_batch, int k, int weight_bits
 
 /* One empty kernel launch (one wave, no instruction but the end of the program). */
 MGEMV_API int mgemv_probe_empty_launch(void *stream);
+/* The same with a grid of `workgroups` workgroups of `waves_per_workgroup` waves (1-16), e.g. the
+ * GEMV's own launch shape: what dispatching that many waves costs before any of them does anything. */
+MGEMV_API int mgemv_probe_empty_grid(int workgroups, int waves_per_workgroup, void *stream);
 
 /* Streams `bytes` of device memory at src (rounded down to whole 4-KiB units per wave) through
  * workgroups x waves_per_workgroup waves, each reading its own contiguous range with the weight

@@ -18,6 +18,7 @@ from .api import (  # noqa: F401
     host_gemv,
     static_scratch_bytes_needed,
     STATIC_SCRATCH_BYTES,
+    probe_empty_grid,
     probe_empty_launch,
     probe_gemv,
     probe_stream_read,

@@ -370,6 +370,12 @@ def probe_empty_launch(stream=None):
     _lib.check(_lib.lib().mgemv_probe_empty_launch(_stream_ptr(stream)), "probe_empty_launch")
 
 
+def probe_empty_grid(workgroups, waves_per_workgroup, stream=None):
+    """An empty kernel with the given grid (mgemv_probe_empty_grid)."""
+    _lib.check(_lib.lib().mgemv_probe_empty_grid(int(workgroups), int(waves_per_workgroup), _stream_ptr(stream)),
+               "probe_empty_grid")
+
+
 def probe_stream_read(src, nbytes, workgroups, waves_per_workgroup, units_in_flight, sink=None, stream=None):
     """Plain streaming read of nbytes at src with the GEMV's weight loads (mgemv_probe_stream_read)."""
     _lib.check(_lib.lib().mgemv_probe_stream_read(_dev_ptr(src), int(nbytes), int(workgroups), int(waves_per_workgroup),

@@ -8,6 +8,7 @@
 namespace mgemv {
 
 __global__ void __launch_bounds__(64) empty_kernel() {}
+__global__ void __launch_bounds__(kWave * kMaxWavesPerWorkgroup) empty_grid_kernel() {}
 
 // Every wave streams its own contiguous range of 4-KiB units with the loads of the GEMV kernel
 // (one 1-KiB block per wave-wide 128-bit load, streaming cache hint), DEPTH units requested
@@ -74,6 +75,15 @@ extern "C" {
 
 int mgemv_probe_empty_launch(void* stream) {
   return mgemv::launch(mgemv::empty_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream)) == hipSuccess
+             ? MGEMV_OK
+             : MGEMV_ERR_LAUNCH;
+}
+
+int mgemv_probe_empty_grid(int workgroups, int waves_per_workgroup, void* stream) {
+  if (workgroups < 1 || workgroups > (1 << 20) || waves_per_workgroup < 1 || waves_per_workgroup > mgemv::kMaxWavesPerWorkgroup)
+    return MGEMV_ERR_SIZE;
+  return mgemv::launch(mgemv::empty_grid_kernel, dim3((unsigned)workgroups), dim3((unsigned)(mgemv::kWave * waves_per_workgroup)),
+                       0, static_cast<hipStream_t>(stream)) == hipSuccess
              ? MGEMV_OK
              : MGEMV_ERR_LAUNCH;
 }

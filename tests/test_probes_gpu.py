@@ -67,7 +67,12 @@ def test_stream_read_and_empty_launch_run_and_check_their_arguments(gpu):
     for wgs, waves, depth in ((256, 4, 2), (64, 16, 4), (8, 1, 8)):
         mg.probe_stream_read(buf, buf.numel(), wgs, waves, depth, sink)
     mg.probe_empty_launch()
+    mg.probe_empty_grid(256, 4)
+    mg.probe_empty_grid(8016, 1)
     torch.cuda.synchronize()
+    for bad in ((0, 4), (256, 0), (256, 17)):
+        with pytest.raises(MixedGemvError):
+            mg.probe_empty_grid(*bad)
     for bad in ((0, 4, 2), (256, 17, 2), (256, 4, 3), (4096, 16, 2)):   # the last: less than one unit per wave
         with pytest.raises(MixedGemvError):
             mg.probe_stream_read(buf, buf.numel(), *bad, sink)
