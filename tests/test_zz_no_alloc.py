@@ -45,3 +45,29 @@ def test_static_scratch_entry_refuses_what_does_not_fit(gpu):
     small = Problem("na_after", 256, 1024, 4, SCALE_AND_ZEROS, 128, bias=True, scale_range=(0.1, 0.3), zero_kind="int8")
     want, got = both(small)
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+
+
+def test_static_scratch_entry_from_several_threads(gpu):
+    """All callers share one device array and one host array; the library serialises them.  Four threads,
+    different problems, three calls each: every result equals the allocating entry's."""
+    import threading
+    probs = [Problem(f"na_t{i}", 128 * (i + 1), 1024 + 512 * i, 4, SCALE_AND_ZEROS, 128, bias=True, scale_range=(0.1, 0.3),
+                     zero_kind="int8") for i in range(4)]
+    want = [mg.host_gemv(p.w_raw, p.x, p.scale, p.zeros_i8, p.bias, 1, p.n_out, 1, p.k, p.group_size, p.quant_op, p.bits)
+            for p in probs]
+    failures = []
+
+    def worker(i):
+        p = probs[i]
+        for _ in range(3):
+            got = mg.host_gemv(p.w_raw, p.x, p.scale, p.zeros_i8, p.bias, 1, p.n_out, 1, p.k, p.group_size, p.quant_op,
+                               p.bits, static_scratch=True)
+            if not np.array_equal(got.view(np.uint16), want[i].view(np.uint16)):
+                failures.append(i)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
