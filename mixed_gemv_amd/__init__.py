@@ -21,6 +21,7 @@ from .api import (  # noqa: F401
     probe_empty_grid,
     probe_empty_launch,
     probe_gemv,
+    probe_gemv_rows,
     probe_stream_read,
     PROBE_COMPUTE_ONLY,
     PROBE_LOADS_ONLY,

@@ -360,6 +360,13 @@ def set_prefetch_stages(stages):
     _lib.check(_lib.lib().mgemv_set_prefetch_stages(int(stages)), "set_prefetch_stages")
 
 
+def probe_gemv_rows(kind, N, ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_D, M, K, group_size, stream=None):
+    """PROBE_LOADS_ONLY / PROBE_COMPUTE_ONLY builds for a launch of N activation rows (mgemv_probe_gemv_rows)."""
+    _lib.check(_lib.lib().mgemv_probe_gemv_rows(int(kind), int(N), _dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale),
+                                                _dev_ptr(ptr_zero_point), _dev_ptr(ptr_D), int(M), int(K), int(group_size),
+                                                _stream_ptr(stream)), "probe_gemv_rows")
+
+
 PROBE_LOADS_ONLY = 1
 PROBE_TIMELINE = 2
 PROBE_COMPUTE_ONLY = 3

@@ -612,6 +612,13 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
     g.tail.y = reinterpret_cast<half_t*>(y);
     g.tail.m_batch = m_batch;
     g.lds = launch_resources(g.plan, weight_bits, m_batch, act).lds_bytes;
+    if (probe != kProbeNone) {
+      const int rounds = g.plan.staged_rows != 0 ? g.plan.staged_rows / g.plan.tiles_per_wg : 0;
+      if (probe == kProbeTimeline || rounds == 0 ||
+          !mfma_lds_probe_exists(weight_bits, quant_op, gpr, rounds, act, g.plan.tiles_per_wg))
+        return MGEMV_ERR_QUANT_OP;
+      return launch_mfma_lds_probe(g, gpr, rounds, probe) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+    }
     if (g.plan.staged_rows != 0) {
       return launch_mfma_lds(g, weight_bits, quant_op, gpr, g.plan.staged_rows / g.plan.tiles_per_wg, act) == hipSuccess
                  ? MGEMV_OK
@@ -716,16 +723,29 @@ int mgemv_dequantize(const void* weights, const uint16_t* scale, const uint16_t*
                                mgemv::kActF16);
 }
 
+namespace {
+int probe_kind(int kind) {
+  return kind == MGEMV_PROBE_LOADS_ONLY     ? mgemv::kProbeLoadsOnly
+         : kind == MGEMV_PROBE_COMPUTE_ONLY ? mgemv::kProbeComputeOnly
+                                            : mgemv::kProbeTimeline;
+}
+}  // namespace
+
+int mgemv_probe_gemv_rows(int kind, int m_batch, const void* weights, const uint16_t* x, const uint16_t* scale,
+                          const uint16_t* zero_add, uint16_t* y, int n_out, int k, int group_size, void* stream) {
+  if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_COMPUTE_ONLY) return MGEMV_ERR_SIZE;
+  return mgemv::gemv_any(weights, x, scale, zero_add, nullptr, y, 1, n_out, m_batch, k, group_size,
+                         MGEMV_FINEGRAINED_SCALE_AND_ZEROS, 4, 0, 0, 0, 0, 0, stream, mgemv::kActF16, 1.0f, 1.0f,
+                         probe_kind(kind), nullptr);
+}
+
 int mgemv_probe_gemv(int kind, unsigned long long* trace, const void* weights, const uint16_t* x, const uint16_t* scale,
                      const uint16_t* zero_add, uint16_t* y, int n_out, int k, int group_size, void* stream) {
   if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_TIMELINE && kind != MGEMV_PROBE_COMPUTE_ONLY) return MGEMV_ERR_SIZE;
   if (kind == MGEMV_PROBE_TIMELINE && (trace == nullptr || reinterpret_cast<uintptr_t>(trace) % 8)) return MGEMV_ERR_NULL_POINTER;
   return mgemv::gemv_any(weights, x, scale, zero_add, nullptr, y, 1, n_out, 1, k, group_size,
                          MGEMV_FINEGRAINED_SCALE_AND_ZEROS, 4, 0, 0, 0, 0, 0, stream, mgemv::kActF16, 1.0f, 1.0f,
-                         kind == MGEMV_PROBE_LOADS_ONLY     ? mgemv::kProbeLoadsOnly
-                         : kind == MGEMV_PROBE_COMPUTE_ONLY ? mgemv::kProbeComputeOnly
-                                                            : mgemv::kProbeTimeline,
-                         trace);
+                         probe_kind(kind), trace);
 }
 
 // gemv/device/gemv_adaptor.h:114-178 as one plain struct.

@@ -237,6 +237,9 @@ hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr);
 hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act);
 // Measurement builds of the single-row int4 scale-and-zero fp16 VALU kernel (probe: kProbeLoadsOnly / kProbeTimeline / kProbeComputeOnly).
 hipError_t launch_gemv_probe(const GemvLaunch& g, int probe);
+// ... and of the LDS-staged matrix-core kernel (kProbeLoadsOnly / kProbeComputeOnly), where they exist.
+bool mfma_lds_probe_exists(int bits, int qop, int gpr, int rounds, int act, int tiles_per_wg);
+hipError_t launch_mfma_lds_probe(const GemvLaunch& g, int gpr, int rounds, int probe);
 
 }  // namespace mgemv
 

@@ -414,10 +414,41 @@ __device__ __forceinline__ void park_x_rows(const XRows<BITS, ROUNDS>& r, uint8_
   }
 }
 
+// Measurement builds.  keep_registers: the compiler must assume that a unit's registers changed (so
+// that repeating its arithmetic is not hoisted out of the loop); no instruction.  consume_unit: every
+// register of the unit and one staged operand have to be there, nothing is computed with them.
+template <int BITS, int GROUPS_PER_RUN, int ROUNDS>
+__device__ __forceinline__ void keep_registers(MfmaWeights<BITS, GROUPS_PER_RUN>& f, XRows<BITS, ROUNDS>& r) {
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) asm volatile("" : "+v"(f.w[i]));
+#pragma unroll
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) asm volatile("" : "+v"(f.s[gi]), "+v"(f.z[gi]));
+#pragma unroll
+  for (int j = 0; j < ROUNDS; ++j)
+#pragma unroll
+    for (int h = 0; h < (BITS == 4 ? 4 : 2); ++h) asm volatile("" : "+v"(r.v[j][h]));
+}
+
+template <int BITS, int GROUPS_PER_RUN>
+__device__ __forceinline__ void consume_unit(f32x4& acc, const MfmaWeights<BITS, GROUPS_PER_RUN>& f,
+                                             const LdsActivations<BITS>& xa) {
+  uint32_t t = 0;
+#pragma unroll
+  for (int i = 0; i < kBlocksPerUnit; ++i) t ^= f.w[i][0] ^ f.w[i][1] ^ f.w[i][2] ^ f.w[i][3];
+#pragma unroll
+  for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) t ^= f.s[gi] ^ f.z[gi];
+  t ^= *reinterpret_cast<const uint32_t*>(xa.lane_base);
+  acc[0] += __builtin_bit_cast(float, t & 0x3fffffffu);
+}
+
 // blockDim = (64 * split_k, tiles_per_wg), at most 8 waves.  Dynamic LDS: split_k * 2 stages of
 // (ROUNDS * tiles_per_wg) rows x kRowStride bytes, then tiles_per_wg * split_k * 256 floats for
 // the split-K combine.
-template <int BITS, int QOP, int GROUPS_PER_RUN, int ROUNDS, int ACT, bool SHARED>
+// PROBE: kProbeNone the product; kProbeLoadsOnly keeps every load, the staging and the barriers and
+// replaces the arithmetic of a unit by taking its registers and one staged operand; kProbeComputeOnly
+// requests only the first k step of a wave's range and repeats the staging and the arithmetic of
+// that step for every further one (measurement builds, wrong results).
+template <int BITS, int QOP, int GROUPS_PER_RUN, int ROUNDS, int ACT, bool SHARED, int PROBE = kProbeNone>
 __global__ void __launch_bounds__(kWave * kMaxWavesPerMfmaWorkgroup)
 gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out,
                      int k, uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
@@ -514,24 +545,40 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
     // even step: weights in wa, stage 0
     park_x_rows<BITS, ROUNDS>(xr, my_stages, lane, ty, p.tiles_per_wg);
     stage_ready();
-    fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin + u + 1, lane, ty, p.tiles_per_wg);
-    load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wb, p, w_rsrc, tables, u + 1, ks_begin + u + 1, lane, row);
+    if constexpr (PROBE == kProbeComputeOnly) {
+      wb = wa;
+      keep_registers(wb, xr);
+    } else {
+      fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin + u + 1, lane, ty, p.tiles_per_wg);
+      load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wb, p, w_rsrc, tables, u + 1, ks_begin + u + 1, lane, row);
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (u < units) {
       const LdsActivations<BITS> xa{my_stages + operand_offset};
-      compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, wa, xa, c, col_scale, short_ok);
+      if constexpr (PROBE == kProbeLoadsOnly)
+        consume_unit(acc, wa, xa);
+      else
+        compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, wa, xa, c, col_scale, short_ok);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (u + 1 < steps) {
       // odd step: weights in wb, stage 1
       park_x_rows<BITS, ROUNDS>(xr, my_stages + stage_bytes, lane, ty, p.tiles_per_wg);
       stage_ready();
-      fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin + u + 2, lane, ty, p.tiles_per_wg);
-      load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wa, p, w_rsrc, tables, u + 2, ks_begin + u + 2, lane, row);
+      if constexpr (PROBE == kProbeComputeOnly) {
+        wa = wb;
+        keep_registers(wa, xr);
+      } else {
+        fetch_x_rows<BITS, ROUNDS>(xr, p, x_rsrc, ks_begin + u + 2, lane, ty, p.tiles_per_wg);
+        load_weights_lds_mfma<BITS, QOP, GROUPS_PER_RUN>(wa, p, w_rsrc, tables, u + 2, ks_begin + u + 2, lane, row);
+      }
       __builtin_amdgcn_sched_barrier(0);
       if (u + 1 < units) {
         const LdsActivations<BITS> xa{my_stages + stage_bytes + operand_offset};
-        compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, wb, xa, c, col_scale, short_ok);
+        if constexpr (PROBE == kProbeLoadsOnly)
+          consume_unit(acc, wb, xa);
+        else
+          compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, wb, xa, c, col_scale, short_ok);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -615,9 +662,9 @@ hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr) {
 }
 
 // LDS-staged matrix-core kernel: 2 tiles per workgroup share the activation stage.
-template <int BITS, int QOP, int GPR, int ROUNDS, int ACT, bool SHARED>
+template <int BITS, int QOP, int GPR, int ROUNDS, int ACT, bool SHARED, int PROBE = kProbeNone>
 hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
-  const auto kernel = gemv_mfma_lds_kernel<BITS, QOP, GPR, ROUNDS, ACT, SHARED>;
+  const auto kernel = gemv_mfma_lds_kernel<BITS, QOP, GPR, ROUNDS, ACT, SHARED, PROBE>;
   if (g.lds > 48 * 1024) {
     // More than 48 KiB of dynamic LDS has to be granted per kernel and device; remember the
     // largest grant so that only the first such launch pays for the call.
@@ -682,6 +729,28 @@ hipError_t launch_mfma_lds_act(const GemvLaunch& g, int bits, int qop, int gpr, 
     case 2: return launch_mfma_lds_gpr<8, 2, ACT>(g, gpr, rounds);
     default: return launch_mfma_lds_gpr<8, 3, ACT>(g, gpr, rounds);
   }
+}
+
+// Measurement builds exist for int4 scale-and-zero fp16 launches whose workgroups share their stages:
+// one or two groups per lane run, 4 or 8 staging rounds per wave (8 or 16 rows over 2 tiles).
+template <int PROBE>
+hipError_t launch_mfma_lds_probe_kind(const GemvLaunch& g, int gpr, int rounds) {
+  constexpr int kQ = MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  if (gpr == 1)
+    return rounds == 4 ? launch_mfma_lds_kernel_r<4, kQ, 1, 4, kActF16, true, PROBE>(g)
+                       : launch_mfma_lds_kernel_r<4, kQ, 1, 8, kActF16, true, PROBE>(g);
+  return rounds == 4 ? launch_mfma_lds_kernel_r<4, kQ, 2, 4, kActF16, true, PROBE>(g)
+                     : launch_mfma_lds_kernel_r<4, kQ, 2, 8, kActF16, true, PROBE>(g);
+}
+
+bool mfma_lds_probe_exists(int bits, int qop, int gpr, int rounds, int act, int tiles_per_wg) {
+  return bits == 4 && qop == MGEMV_FINEGRAINED_SCALE_AND_ZEROS && (gpr == 1 || gpr == 2) && (rounds == 4 || rounds == 8) &&
+         act == kActF16 && tiles_per_wg > 1;
+}
+
+hipError_t launch_mfma_lds_probe(const GemvLaunch& g, int gpr, int rounds, int probe) {
+  return probe == kProbeLoadsOnly ? launch_mfma_lds_probe_kind<kProbeLoadsOnly>(g, gpr, rounds)
+                                  : launch_mfma_lds_probe_kind<kProbeComputeOnly>(g, gpr, rounds);
 }
 
 hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act) {

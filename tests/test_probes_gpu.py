@@ -60,6 +60,27 @@ def test_compute_only_build_repeats_the_first_unit(gpu, n_out, k, split):
         mg.set_launch_override(0, 0, 0, 0)
 
 
+@pytest.mark.parametrize("m_batch", [4, 8, 16])
+def test_matrix_core_measurement_builds_run(gpu, m_batch):
+    """Loads-only and arithmetic-only builds of the LDS-staged matrix-core kernel: they exist for launches
+    whose workgroups share a stage between tiles, write every output, and are refused elsewhere."""
+    import torch
+    n_out, k = 8192, 2048       # 512 tiles: two tiles per workgroup
+    prob = Problem("probe_mc", n_out, k, 4, SCALE_AND_ZEROS, 64, m_batch=m_batch, x_dist="normal")
+    dev = DeviceProblem(prob, gpu)
+    plan = mg.query_launch(n_out, m_batch, k, 4, 64)
+    assert plan["matrix_core"] == 2 and plan["tiles_per_wg"] >= 2
+    for kind in (mg.PROBE_LOADS_ONLY, mg.PROBE_COMPUTE_ONLY):
+        dev.y.fill_(0x7e00)
+        mg.probe_gemv_rows(kind, m_batch, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 64)
+        torch.cuda.synchronize()
+        assert not np.any(dev.y.cpu().numpy().view(np.uint16) == 0x7e00)
+    with pytest.raises(MixedGemvError):     # one tile per workgroup: no measurement build
+        mg.probe_gemv_rows(mg.PROBE_LOADS_ONLY, 8, dev.w, dev.x, dev.scale, dev.zero, dev.y, 2048, k, 64)
+    with pytest.raises(MixedGemvError):
+        mg.probe_gemv_rows(mg.PROBE_TIMELINE, 8, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 64)
+
+
 def test_stream_read_and_empty_launch_run_and_check_their_arguments(gpu):
     import torch
     buf = torch.zeros(8 << 20, dtype=torch.uint8, device=gpu)
