@@ -63,6 +63,62 @@ def measured_traffic_bytes(name, m_batch):
     return int((fetch * FETCH_SCALE + write * WRITE_SCALE) * 1024)
 
 
+def measure_traffic_live(name, log=None):
+    """HBM bytes per launch of workload `name`, measured now: four short child runs of this file under
+    `rocprofv3 --pmc` (FETCH_SIZE and WRITE_SIZE of the workload's kernel, then of a 512 MiB device copy
+    that calibrates the two counters).  Returns (bytes, description) or (None, reason)."""
+    import csv
+    import glob
+    import shutil
+    import subprocess
+    import tempfile
+    tool = shutil.which("rocprofv3")
+    if tool is None:
+        return None, "rocprofv3 not found"
+    if any(k.startswith("ROCPROF") or k.startswith("ROCP_") for k in os.environ):
+        return None, "this run is itself being profiled"
+    here = os.path.abspath(__file__)
+    steps = {"ns": 140}.get(name, 64)
+    work = ["--workload", name, "--no-cpu", "--no-ceilings", "--no-warm-cache", "--no-traffic", "--extra", "",
+            "--steps", str(steps), "--warmup", "8", "--launch", "stream"]
+    runs = (("FETCH_SIZE", work, ("gemv_dpp_kernel", "gemv_mfma")), ("WRITE_SIZE", work, ("gemv_dpp_kernel", "gemv_mfma")),
+            ("FETCH_SIZE", ["--copy-calibration"], ("copyBuffer",)), ("WRITE_SIZE", ["--copy-calibration"], ("copyBuffer",)))
+    values = []
+    tmp = tempfile.mkdtemp(prefix="mgemv_pmc_", dir="/tmp")
+    try:
+        env = dict(os.environ, TMPDIR="/tmp")
+        for i, (counter, args, kernels) in enumerate(runs):
+            out_dir = os.path.join(tmp, f"run{i}")
+            cmd = [tool, "--pmc", counter, "--output-format", "csv", "-d", out_dir, "--", sys.executable, here] + args
+            try:
+                proc = subprocess.run(cmd, cwd="/tmp", env=env, capture_output=True, text=True, timeout=150)
+            except subprocess.TimeoutExpired:
+                return None, f"the {counter} pass did not finish in 150 s"
+            if proc.returncode != 0:
+                return None, f"the {counter} pass ended with status {proc.returncode}"
+            got = []
+            for f in glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True):
+                with open(f) as fh:
+                    for row in csv.DictReader(fh):
+                        if row.get("Counter_Name") == counter and any(k in row.get("Kernel_Name", "") for k in kernels):
+                            got.append(float(row["Counter_Value"]))
+            if not got:
+                return None, f"the {counter} pass recorded no dispatch of the kernel"
+            got = got[len(got) // 4:] or got
+            values.append((sum(got) / len(got), len(got)))
+            if log:
+                log(f"traffic pass {i}: {counter} = {values[-1][0]:.1f} KiB per dispatch over {values[-1][1]} dispatches")
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
+    (fetch, n_f), (write, _), (copy_fetch, _), (copy_write, _) = values
+    copied_kib = (512 << 20) / 1024.0
+    fetch_scale, write_scale = copied_kib / copy_fetch, copied_kib / copy_write
+    total = int((fetch * fetch_scale + write * write_scale) * 1024)
+    return total, (f"measured by this run: rocprofv3 --pmc FETCH_SIZE {fetch:.1f} and WRITE_SIZE {write:.1f} KiB per dispatch "
+                   f"(child runs of this file, --workload {name} --launch stream, {n_f} dispatches), scaled by what the same "
+                   f"counters read for a 512 MiB device copy (x {fetch_scale:.3f}, x {write_scale:.3f})")
+
+
 def algorithmic_bytes(n_out, k, bits, quant_op, group, m_batch, bias):
     groups = 1 if quant_op == 1 else k // group
     return (n_out * k * bits // 8 + groups * n_out * 2 * (2 if quant_op == 3 else 1) + (n_out * 2 if bias else 0)
@@ -555,6 +611,9 @@ def main():
     ap.add_argument("--no-ceilings", action="store_true",
                     help="skip the ceiling measurements (plain streaming reads, the kernel without its arithmetic, "
                          "the timeline of one launch)")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="do not measure the headline kernel's HBM traffic with rocprofv3 child runs (about a minute); "
+                         "roofline.traffic then carries the figure of the committed profile")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only copy 512 MiB device to device four times and exit: the known-size kernel against which "
                          "the FETCH_SIZE / WRITE_SIZE counters of `rocprofv3 --pmc` are scaled")
@@ -563,6 +622,11 @@ def main():
         print("bench.py: this build measures one GPU only (a GEMV over one weight matrix held by one MI355X); "
               "--gpus above 1 is not supported", file=sys.stderr)
         sys.exit(2)
+
+    # the counter passes run first, as children, before this process touches the GPU
+    live_traffic = (None, "not asked for")
+    if not args.no_traffic and not args.copy_calibration and (args.m_batch in (None, 1)):
+        live_traffic = measure_traffic_live(args.workload, log=lambda t: print(t, file=sys.stderr, flush=True))
 
     import torch
     if not torch.cuda.is_available():
@@ -620,9 +684,11 @@ def main():
         "pct_of_hbm_peak": round(100.0 * m["value_GBps"] / HBM_PEAK_GBS, 2),
         "algorithmic_bytes_per_call": wl.bytes,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic_bytes(wl.name, wl.m_batch),
-                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this workload, "
-                                       "scaled by a 512 MiB copy (profiles/); not re-measured by this run",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": live_traffic[0] if live_traffic[0] is not None else measured_traffic_bytes(wl.name, wl.m_batch),
+                     "traffic_source": live_traffic[1] if live_traffic[0] is not None else (
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this workload, scaled by a 512 MiB "
+                         "copy (profiles/); not re-measured by this run: " + live_traffic[1]),
                      "kernel_us_avg_events": kernel_us, "kernel_us_measured_over_steps": long_steps,
                      "kernel_us_avg_events_timed_region": m["kernel_us_avg_events"]},
     }
