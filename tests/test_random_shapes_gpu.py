@@ -32,6 +32,15 @@ def _cases():
             element = "bf16" if rng.random() < 0.35 else "f16"
             out.append((f"r{len(out)}_{n_out}x{k}_i{bits}_q{qop}_g{group}_m{m_batch}_{element}",
                         n_out, k, bits, qop, group, m_batch, bool(rng.integers(0, 2)), element))
+    # per-column mode with reductions that are a multiple of 8 only (utils/preprocess.h:324-327)
+    for _ in range(8):
+        bits = int(rng.choice([4, 8]))
+        n_out = int(rng.integers(1, 200)) * 4
+        k = int(rng.integers(1, 400)) * 8
+        m_batch = int(rng.choice([1, 2, 4, 5, 8, 16]))
+        element = "bf16" if rng.random() < 0.35 else "f16"
+        out.append((f"r{len(out)}_{n_out}x{k}_i{bits}_q1_g0_m{m_batch}_{element}", n_out, k, bits, PER_COLUMN, 0, m_batch,
+                    bool(rng.integers(0, 2)), element))
     # enough tiles for 8 of them to share one 16-row activation stage, and for 2 to share 8 rows
     out.append(("fixed_21780x160_i4_q3_g160_m13_f16", 21780, 160, 4, SCALE_AND_ZEROS, 160, 13, True, "f16"))
     out.append(("fixed_22000x128_i4_q2_g64_m16_bf16", 22000, 128, 4, SCALE_ONLY, 64, 16, False, "bf16"))
