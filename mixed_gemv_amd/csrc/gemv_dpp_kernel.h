@@ -354,7 +354,9 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   // The library is built with kernel-argument preloading: the four pointers and six words in
   // front of GemvTail arrive in SGPRs with the wave (firmware without the feature runs a short
   // prologue that loads them instead).  Nothing on the way to the first weight loads of an
-  // unbatched launch reads the tail, so those loads do not wait for any scalar load at all.
+  // unbatched launch whose waves stay on one tile reads the tail, so those loads do not wait
+  // for any scalar load at all: `tail` itself is only touched by batched launches and tile
+  // walks, everything else reads the copy `late`, fetched once the first unit is requested.
   // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223): problems past the first fetch
   // their strides first.
   const long long batch = blockIdx.z;
@@ -364,9 +366,6 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     p.scale += batch * tail.stride_scale;
     p.zero_add += batch * tail.stride_scale;  // only dereferenced in scale+zero mode
   }
-  const bool has_bias = tail.bias != nullptr;
-  tail.bias += batch * tail.stride_bias;
-  tail.y += batch * tail.stride_y;
 
   const int wg = logical_workgroup(p);
   if (wg >= p.workgroups) return;  // whole workgroup leaves before any barrier
@@ -374,14 +373,14 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   const int lane = threadIdx.x % kWave;
   const int kw = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // position along k
   const int ty = __builtin_amdgcn_readfirstlane(threadIdx.y);         // tile sequence within the workgroup
-  const int split_k = tail.split_k;
   const int tiles = (p.n_out + kTileRows - 1) / kTileRows;
   // The host's launch geometry leaves no wave without units (split_k = ceil(ksteps / steps_per_wave)).
-  const WaveWork work = valu_wave_work(MULTI, wg, ty, kw, p.tiles_per_wg, tail.seq_base, tail.seq_rem, tiles,
-                                       p.steps_per_wave, p.ksteps);
+  const WaveWork work = valu_wave_work(MULTI, wg, ty, kw, p.tiles_per_wg, MULTI ? tail.seq_base : 0,
+                                       MULTI ? tail.seq_rem : 0, tiles, p.steps_per_wave, p.ksteps);
   const int tile_begin = work.tile_begin, my_tiles = work.tiles, ks_begin = work.ks_begin, units = work.units;
-  const int park_stride = p.tiles_per_wg * split_k * MB * kWave;  // floats between consecutive tiles of a sequence
 
+  GemvTail late;
+  if (my_tiles <= 0) late = read_tail_here();
   if (my_tiles > 0) {
     const int total = MULTI ? my_tiles * units : units;
     const int tile_stride = p.ksteps * kUnitBytes;
@@ -403,7 +402,6 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
 #pragma unroll
     for (int m = 0; m < MB; ++m) acc[m] = 0.0f;
     int pending = units;     // MULTI: units of the current tile still to compute
-    float* slot = partials + (ty * split_k + kw) * MB * kWave + lane;  // MULTI
 
     // Two fragments in flight: the loads of unit u+1 are issued before unit u is computed, so
     // a wave that is waiting for its turn on the VALU still has memory requests outstanding.
@@ -412,6 +410,10 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     // fragments inside, without that wait, measured the same to 2 % on every shape.)
     UnitFragment<BITS, MB, GROUPS_PER_RUN> fa, fb;
     load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fa, p, w_rsrc, x_rsrc, tables, cur);
+    __builtin_amdgcn_sched_barrier(0);
+    late = read_tail_here();
+    const int park_stride = p.tiles_per_wg * late.split_k * MB * kWave;  // floats between consecutive tiles of a sequence
+    float* slot = partials + (ty * late.split_k + kw) * MB * kWave + lane;  // MULTI
     if constexpr (PROBE == kProbeTimeline) {
       __builtin_amdgcn_sched_barrier(0);
       stamp[1] = __builtin_amdgcn_s_memrealtime();      // the first unit is requested
@@ -420,7 +422,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (PROBE == kProbeComputeOnly) fb = fa;  // (waits for the first unit; every later "load" re-uses it)
-    const bool short_ok = (tail.flags & kExactIntegerFormOnly) == 0;
+    const bool short_ok = (late.flags & kExactIntegerFormOnly) == 0;
     const ConvertRegs c = make_convert_regs();
     // With two or more activation rows, a wave of exactly two units runs straight-line code: the
     // second unit is requested without waiting for the first and nothing is prefetched past the
@@ -448,7 +450,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       // 263-352) is this one.  With the single-stage flag every prefetch is waited for as soon as it is
       // issued, which gives that behaviour -- loads and arithmetic strictly one after the other -- to the
       // same code; results do not change.
-      const bool single_stage = (tail.flags & kSingleStage) != 0;
+      const bool single_stage = (late.flags & kSingleStage) != 0;
       int u = 0;
       do {
         advance<MULTI>(cur, walk);
@@ -488,8 +490,13 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       stamp[3] = __builtin_amdgcn_s_memrealtime();      // the last unit is computed
       __builtin_amdgcn_sched_barrier(0);
     }
-    if constexpr (!MULTI) finish_tile<MB>(acc, partials + (ty * split_k + kw) * MB * kWave + lane_after_loop());
+    if constexpr (!MULTI) finish_tile<MB>(acc, partials + (ty * late.split_k + kw) * MB * kWave + lane_after_loop());
   }
+  const int split_k = late.split_k;
+  const int park_stride = p.tiles_per_wg * split_k * MB * kWave;
+  const bool has_bias = late.bias != nullptr;
+  late.bias += batch * late.stride_bias;
+  late.y += batch * late.stride_y;
 
   // Split-K combine (gemv/threadblock/accumulator_combine.h:269-329): every wave has parked
   // its 64 per-lane partial sums of each tile in LDS; after ONE barrier the (tile, activation
@@ -509,13 +516,13 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       sum = (((sum + a0) + a1) + a2) + a3;
     }
     for (; w < split_k; ++w) sum += part[w * MB * kWave];
-    store_outputs<ACT>(tail, has_bias, p.n_out, m, tile_begin + j, lane_c, reduce_k_slices(sum));
+    store_outputs<ACT>(late, has_bias, p.n_out, m, tile_begin + j, lane_c, reduce_k_slices(sum));
   }
   if constexpr (PROBE == kProbeTimeline) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // the outputs are on their way
     stamp[4] = __builtin_amdgcn_s_memrealtime();
-    if (tail.trace != nullptr && lane_c == 0) {
-      unsigned long long* out = tail.trace + ((size_t)blockIdx.x * (blockDim.x * blockDim.y / kWave) + ty * split_k + kw) * 5;
+    if (late.trace != nullptr && lane_c == 0) {
+      unsigned long long* out = late.trace + ((size_t)blockIdx.x * (blockDim.x * blockDim.y / kWave) + ty * split_k + kw) * 5;
 #pragma unroll
       for (int i = 0; i < 5; ++i) out[i] = stamp[i];
     }

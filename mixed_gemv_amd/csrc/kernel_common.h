@@ -185,6 +185,28 @@ __device__ __forceinline__ float reduce_k_slices(float v) {
   return v;
 }
 
+// The kernel arguments behind the preloaded ones, read where the caller stands instead of at the
+// kernel's entry.  A by-value kernel argument is fetched by scalar loads that the compiler puts
+// in front of everything else, and as soon as one of the registers they target is needed for
+// something else the wave waits for them -- a miss of the (just invalidated) scalar cache on the way
+// to the first weight loads.  Reading the words through the kernarg segment pointer behind a
+// statement the compiler cannot look through keeps those loads where they are written.
+// The ten arguments in front of the tail occupy 56 bytes in every kernel of this library.
+constexpr int kTailKernargOffset = 56;
+static_assert(alignof(GemvTail) == 8 && kTailKernargOffset % alignof(GemvTail) == 0 && sizeof(GemvTail) % 4 == 0,
+              "GemvTail follows four pointers and six 32-bit words without padding");
+__device__ __forceinline__ GemvTail read_tail_here() {
+  typedef const __attribute__((address_space(4))) uint32_t* KernargWords;
+  KernargWords words = (KernargWords)__builtin_amdgcn_kernarg_segment_ptr() + kTailKernargOffset / 4;
+  asm volatile("" : "+s"(words) : : "memory");
+  uint32_t raw[sizeof(GemvTail) / 4];
+#pragma unroll
+  for (int i = 0; i < (int)(sizeof(GemvTail) / 4); ++i) raw[i] = words[i];
+  GemvTail t;
+  __builtin_memcpy(&t, raw, sizeof(GemvTail));
+  return t;
+}
+
 // The lane number, recomputed.  Used behind the unit loop so that the value computed in front
 // of it need not stay in a register (or be spilled) across the loop.
 __device__ __forceinline__ int lane_after_loop() {
