@@ -70,6 +70,7 @@ def measure_traffic_live(name, log=None):
     import csv
     import glob
     import shutil
+    import signal
     import subprocess
     import tempfile
     tool = shutil.which("rocprofv3")
@@ -90,12 +91,25 @@ def measure_traffic_live(name, log=None):
         for i, (counter, args, kernels) in enumerate(runs):
             out_dir = os.path.join(tmp, f"run{i}")
             cmd = [tool, "--pmc", counter, "--output-format", "csv", "-d", out_dir, "--", sys.executable, here] + args
+            # The profiler starts the python child itself: the pass runs in a session of its own, so that
+            # whatever happens every process of it -- the profiler, its child, their helpers -- can be ended
+            # as one group and is waited for before this function returns.
+            proc = subprocess.Popen(cmd, cwd="/tmp", env=env, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                                    start_new_session=True)
             try:
-                proc = subprocess.run(cmd, cwd="/tmp", env=env, capture_output=True, text=True, timeout=150)
+                status = proc.wait(timeout=150)
             except subprocess.TimeoutExpired:
+                status = None
+            finally:
+                try:
+                    os.killpg(proc.pid, signal.SIGKILL)     # stragglers of a pass that has ended, or the whole pass after a time-out
+                except (ProcessLookupError, PermissionError):
+                    pass
+                proc.wait()
+            if status is None:
                 return None, f"the {counter} pass did not finish in 150 s"
-            if proc.returncode != 0:
-                return None, f"the {counter} pass ended with status {proc.returncode}"
+            if status != 0:
+                return None, f"the {counter} pass ended with status {status}"
             got = []
             for f in glob.glob(os.path.join(out_dir, "**", "*counter_collection.csv"), recursive=True):
                 with open(f) as fh:
@@ -386,8 +400,9 @@ def ceilings_of(wl, use_graph, timeline=False):
                     no arithmetic): us per launch and GB/s of the bytes read;
       loads_only    the GEMV kernel itself with every load kept and the arithmetic removed;
       compute_only  the GEMV kernel itself with the arithmetic kept and only each wave's first unit loaded;
-      timeline      (headline only) when the phases of one launch happen."""
+      timeline      when the phases of one launch happen, and how long its waves wait for their loads."""
     import statistics
+    import numpy as np
     import torch
     import mixed_gemv_amd as mg
     if wl.bits != 4 or wl.quant_op != 3 or wl.m_batch != 1:
@@ -430,35 +445,68 @@ def ceilings_of(wl, use_graph, timeline=False):
                            "note": "the GEMV kernel with its arithmetic kept (dequantise + dot of every unit, combine, store) "
                                    "and only the first unit of each wave loaded"}
     if timeline:
-        n_waves = plan["workgroups"] * waves
-        trace = torch.zeros((n_waves, 5), dtype=torch.int64, device=wl.y.device)
-        rows = []
-        for i in range(40):
+        cus = torch.cuda.get_device_properties(wl.y.device).multi_processor_count
+        plan_dev = mg.query_launch(wl.n_out, 1, wl.k, 4, wl.group, num_compute_units=cus)
+        n_waves = -(-plan_dev["workgroups"] // 8) * 8 * (plan_dev["threads"] // 64)   # the grid is a multiple of 8 workgroups
+        words = mg.PROBE_TIMELINE_WORDS
+        trace = torch.zeros((n_waves, words), dtype=torch.int64, device=wl.y.device)
+        waves = plan_dev["threads"] // 64
+        light, heavy = [], []
+        med = lambda v: float(np.median(v))  # noqa: E731
+        for i in range(48):
             trace.zero_()
             torch.cuda.synchronize()
             # behind a few ordinary launches, so that the probe launch meets the queue as a timed step does
             for w in range(3):
                 wl.launch(i + w)
             j = (i + 3) % wl.sets
-            mg.probe_gemv(mg.PROBE_TIMELINE, trace, wl.w[j], wl.x, wl.s[j], wl.z[j], wl.y, wl.n_out, wl.k, wl.group)
+            # odd passes time the wait in front of every unit as well (two more clock readings per unit, a few per cent slower)
+            mg.probe_gemv(mg.PROBE_TIMELINE_WAITS if i % 2 else mg.PROBE_TIMELINE, trace, wl.w[j], wl.x, wl.s[j], wl.z[j],
+                          wl.y, wl.n_out, wl.k, wl.group)
             torch.cuda.synchronize()
             t = trace.cpu().numpy().astype("float64")
-            t = t[t[:, 0] > 0]
-            if len(t) == 0:
+            if i < 8 or not np.all((t[:, 0] > 0) & (t[:, 11] > 0)):   # (a workgroup without a tile leaves no stamps)
                 continue
             t0 = t[:, 0].min()
-            med = lambda v: float(statistics.median(v))  # noqa: E731
-            rows.append([med(t[:, 0] - t0), float((t[:, 0] - t0).max()), med(t[:, 1] - t[:, 0]), med(t[:, 2] - t[:, 1]),
-                         med(t[:, 3] - t[:, 2]), med(t[:, 4] - t[:, 3]), float(t[:, 4].max() - t0)])
-        if rows:
-            tick_us = 0.01  # s_memrealtime counts a constant 100 MHz clock
-            col = lambda c: round(statistics.median(r[c] for r in rows[5:] or rows) * tick_us, 3)  # noqa: E731
+            if i % 2 == 0:
+                end = t[:, 4] - t0
+                loop_end = (t[:, 3] - t0).reshape(-1, waves)          # by position in the workgroup
+                light.append([med(t[:, 0] - t0), float((t[:, 0] - t0).max()), med(t[:, 1] - t[:, 0]), med(t[:, 2] - t[:, 1]),
+                              med(t[:, 3] - t[:, 2]), med(t[:, 4] - t[:, 3]), float(end.max()), med(end),
+                              float(np.percentile(end, 5)), float(np.percentile(end, 95)),
+                              med((t[:, 13] - t[:, 12]) / np.maximum(t[:, 4] - t[:, 0], 1.0)) * 0.1, med(t[:, 11])]
+                             + [med(loop_end[:, w]) for w in range(waves)])
+            else:
+                waits = t[:, 5:8]
+                b1 = np.where(t[:, 9] > 0, t[:, 9], t[:, 3])
+                b2 = np.where(t[:, 10] > 0, t[:, 10], t[:, 3])
+                spans = np.stack([b1 - t[:, 1], b2 - b1, t[:, 3] - b2], axis=1)   # the thirds of a wave's units
+                heavy.append([med(t[:, 3] - t[:, 1]), med(waits.sum(axis=1)), med(t[:, 8])]
+                             + [v for k3 in range(3) for v in (med(spans[:, k3]), med(waits[:, k3]))])
+        tick_us = 0.01  # s_memrealtime counts a constant 100 MHz clock
+        if light:
+            col = lambda c, rows=light: round(statistics.median(r[c] for r in rows) * tick_us, 3)  # noqa: E731
             out["timeline_us"] = {
                 "clock": "s_memrealtime, 100 MHz (10 ns per tick); medians over the waves of a launch, then over launches",
                 "wave_start_after_first_wave_median": col(0), "wave_start_after_first_wave_last": col(1),
                 "start_to_first_unit_requested": col(2), "requested_to_first_block_arrived": col(3),
                 "first_block_to_last_unit_computed": col(4), "last_unit_to_outputs_stored": col(5),
-                "first_wave_start_to_last_store": col(6), "waves": n_waves, "launches": len(rows)}
+                "first_wave_start_to_last_store": col(6),
+                "wave_end_after_first_wave_start": {"median": col(7), "p5": col(8), "p95": col(9), "last": col(6)},
+                "last_unit_computed_by_wave_of_the_workgroup": [col(12 + w) for w in range(waves)],
+                "units_per_wave": light[-1][11],
+                "shader_clock_GHz": round(statistics.median(r[10] for r in light), 3),
+                "shader_clock_note": "s_memtime ticks per s_memrealtime tick over a wave's life: the clock the compute units "
+                                     "ran at during the probe launch (the power management lowers it under load)",
+                "waves": n_waves, "launches": len(light)}
+            if heavy:
+                col = lambda c, rows=heavy: round(statistics.median(r[c] for r in rows) * tick_us, 3)  # noqa: E731
+                out["timeline_us"]["unit_loop"] = {
+                    "length": col(0), "waiting_in_front_of_units": col(1), "longest_single_wait": col(2),
+                    "by_third_of_units": [{"third": k3 + 1, "length": col(3 + 2 * k3), "waiting": col(4 + 2 * k3)} for k3 in range(3)],
+                    "note": "from the build that also times the explicit wait in front of every unit (operands and first weight "
+                            "block of the unit); what is left of the loop is arithmetic, which the waves of a SIMD share, and "
+                            "the waits for a unit's later blocks inside it"}
     return out
 
 
@@ -663,8 +711,10 @@ def main():
     # not pass for kernel time when the timed region is as short as 20 steps.
     long_steps = max(args.steps, 1000)
     m_long = m if long_steps == args.steps else measure(wl, long_steps, 0, use_graph)
-    kernel_us = m_long["kernel_us_avg_events"]
+    kernel_us_long = m_long["kernel_us_avg_events"]
+    kernel_us = m["kernel_us_avg_events"]          # HIP events round the timed region itself: what the roofline is priced at
     achieved = wl.bytes / (kernel_us * 1e-6) / 1e9
+    achieved_long = wl.bytes / (kernel_us_long * 1e-6) / 1e9
 
     out = {
         "metric": "HBM GB/s & % of peak, us/call; int4-g128 GEMV M=1, N=K=4096",
@@ -698,8 +748,13 @@ def main():
                      "traffic_source": live_traffic[1] if live_traffic[0] is not None else (
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this workload, scaled by a 512 MiB "
                          "copy (profiles/); not re-measured by this run: " + live_traffic[1]),
-                     "kernel_us_avg_events": kernel_us, "kernel_us_measured_over_steps": long_steps,
-                     "kernel_us_avg_events_timed_region": m["kernel_us_avg_events"]},
+                     "kernel_us_avg_events": kernel_us, "kernel_us_measured_over_steps": args.steps,
+                     "note": "achieved / frac: algorithmic bytes over the kernel's average duration by HIP events round the timed "
+                             "region of exactly `steps` launches; a region of 20 launches also carries the start of its graph "
+                             "replay (0.3-0.5 us per launch), which the *_long_region figures, from regions of at least 1000 "
+                             "launches, do not",
+                     "kernel_us_avg_events_long_region": kernel_us_long, "long_region_steps": long_steps,
+                     "achieved_long_region": round(achieved_long, 1), "frac_long_region": round(achieved_long / HBM_PEAK_GBS, 4)},
     }
     # the same launches on ONE buffer set, i.e. out of the Infinity Cache: reported beside the cold
     # figure, never as `value`
@@ -711,7 +766,7 @@ def main():
                              "note": "one buffer set re-read from the 256 MB Infinity Cache; not an HBM figure"}
         floor = launch_floor_us(use_graph)
         out["launch_floor"] = {"us_per_launch": round(floor, 3),
-                               "kernel_us_above_floor": round(kernel_us - floor, 3),
+                               "kernel_us_above_floor": round(kernel_us_long - floor, 3),
                                "note": "cadence of an empty kernel (mgemv_probe_empty_launch) launched like the timed steps"}
     if not args.no_ceilings:
         out["ceilings"] = {wl.name: ceilings_of(wl, use_graph, timeline=True)}
@@ -728,6 +783,7 @@ def main():
             "sample": f"the same loop with OpenMP over the rows, mean of {cpu['all_reps']} runs",
             "us_per_call": round(cpu["all_seconds"] * 1e6, 1)}
         out["parity"] = parity_summary(wl, [0], threads)
+    wl_name = wl.name
     del wl
     torch.cuda.empty_cache()
 
@@ -762,7 +818,7 @@ def main():
             sets = list(range(w2.sets)) if base == "c5" else [0]
             entry["parity"] = parity_summary(w2, sets, threads, with_dequant=(rows in (None, 1)))
         if base == "c5" and element == "f16" and batch == 1 and not args.no_ceilings:
-            out.setdefault("ceilings", {})[base] = ceilings_of(w2, use_graph)
+            out.setdefault("ceilings", {})[base] = ceilings_of(w2, use_graph, timeline=True)
         if base == "c4" and rows in (8, 16) and element == "f16" and batch == 1 and not args.no_ceilings:
             c = ceilings_of_rows(w2, use_graph)
             if c is not None:
@@ -770,6 +826,13 @@ def main():
         others[name] = entry
     built.clear()
     torch.cuda.empty_cache()
+    # every BASELINE entry at a glance: name -> [kernel us by events, fraction of the HBM peak, parity ok (1 / 0, -1 = not checked)]
+    by_workload = {wl_name: [round(kernel_us, 3), round(achieved / HBM_PEAK_GBS, 4),
+                             -1 if "parity" not in out else int(bool(out["parity"].get("ok")))]}
+    for name, e in others.items():
+        by_workload[name] = [e["kernel_us_avg_events"], e["roofline_frac"],
+                             -1 if "parity" not in e else int(bool(e["parity"].get("ok")))]
+    out["roofline"]["by_workload"] = by_workload
     if others:
         out["other_workloads"] = others
         out["all_parity_ok"] = bool(out.get("parity", {}).get("ok", True)

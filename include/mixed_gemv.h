@@ -384,55 +384,6 @@ MGEMV_API int mgemv_query_launch_for(int n_out, int m_batch, int k, int weight_b
 MGEMV_API int mgemv_plan_coverage(int n_out, int m_batch, int k, int weight_bits, int group_size, int element,
                                   int num_compute_units, int64_t out[8]);
 
-/* ------------------------------------------------------------------------------------------
- * Measurement probes.  No counterpart in the reference and not on any product path: they are
- * what the benchmark's "ceilings" are measured with, so that a figure such as "this launch
- * shape cannot read faster than X" is a kernel anybody can run, not a remark.
- * ---------------------------------------------------------------------------------------- */
-
-/* One empty kernel launch (one wave, no instruction but the end of the program). */
-MGEMV_API int mgemv_probe_empty_launch(void *stream);
-/* The same with a grid of `workgroups` workgroups of `waves_per_workgroup` waves (1-16), e.g. the
- * GEMV's own launch shape: what dispatching that many waves costs before any of them does anything. */
-MGEMV_API int mgemv_probe_empty_grid(int workgroups, int waves_per_workgroup, void *stream);
-
-/* Streams `bytes` of device memory at src (rounded down to whole 4-KiB units per wave) through
- * workgroups x waves_per_workgroup waves, each reading its own contiguous range with the weight
- * loads of the GEMV kernel (1 KiB per wave-wide 128-bit load, streaming cache hint) and
- * units_in_flight (2, 4 or 8) 4-KiB units requested ahead; the data is folded into an
- * exclusive-or and dropped.  sink: 4 writable bytes or NULL. */
-MGEMV_API int mgemv_probe_stream_read(const void *src, size_t bytes, int workgroups, int waves_per_workgroup,
-                                      int units_in_flight, uint32_t *sink, void *stream);
-
-/* Measurement builds of the single-row int4 scale-and-zero fp16 GEMV kernel (one group per lane
- * run: group sizes that are multiples of 128), launched with the geometry mgemv_gemv would use:
- *   MGEMV_PROBE_LOADS_ONLY  every load of the kernel, the arithmetic of a unit replaced by an
- *                           exclusive-or over its registers; y receives meaningless values;
- *   MGEMV_PROBE_TIMELINE    the kernel as it is, plus five timestamps per wave from the
- *                           100 MHz constant clock (s_memrealtime), written to trace[wave * 5 + i]
- *                           (wave = workgroup * waves per workgroup + wave in workgroup; workgroups
- *                           and threads as mgemv_query_launch reports): i = 0 the wave starts,
- *                           1 its first unit is requested, 2 that unit's first block has arrived,
- *                           3 its last unit is computed, 4 its outputs are stored.  y is the
- *                           GEMV's result;
- *   MGEMV_PROBE_COMPUTE_ONLY every wave loads the first unit of its range and then runs the
- *                           arithmetic of that unit once per unit of the range, loading nothing
- *                           more: what the kernel's instructions alone take; y is meaningless. */
-enum { MGEMV_PROBE_LOADS_ONLY = 1, MGEMV_PROBE_TIMELINE = 2, MGEMV_PROBE_COMPUTE_ONLY = 3 };
-MGEMV_API int mgemv_probe_gemv(int kind, unsigned long long *trace, const void *weights, const uint16_t *x,
-                               const uint16_t *scale, const uint16_t *zero_add, uint16_t *y, int n_out, int k,
-                               int group_size, void *stream);
-
-/* The same two builds -- MGEMV_PROBE_LOADS_ONLY, MGEMV_PROBE_COMPUTE_ONLY -- for a launch of m_batch
- * activation rows, where they exist: one row as above; on the matrix cores the LDS-staged kernel whose
- * workgroups share their activation stage between two or more tiles (int4, scale and zero, fp16,
- * group sizes 64-512; e.g. 8192 x 8192 at 4-16 rows).  There "loads only" keeps the staging of the
- * activation rows and the barriers, and "compute only" requests a wave's first k step only and
- * repeats that step's staging and arithmetic.  Other launches return MGEMV_ERR_QUANT_OP. */
-MGEMV_API int mgemv_probe_gemv_rows(int kind, int m_batch, const void *weights, const uint16_t *x,
-                                    const uint16_t *scale, const uint16_t *zero_add, uint16_t *y, int n_out, int k,
-                                    int group_size, void *stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,8 @@ from .api import (  # noqa: F401
     PROBE_COMPUTE_ONLY,
     PROBE_LOADS_ONLY,
     PROBE_TIMELINE,
+    PROBE_TIMELINE_WAITS,
+    PROBE_TIMELINE_WORDS,
     preprocessed_size,
     plan_coverage,
     query_launch,

@@ -46,7 +46,7 @@ SIGNATURES = {
     "mgemv_probe_empty_launch": (_c.c_int, [_vp]),
     "mgemv_probe_empty_grid": (_c.c_int, [_c.c_int, _c.c_int, _vp]),
     "mgemv_probe_stream_read": (_c.c_int, [_vp, _c.c_size_t, _c.c_int, _c.c_int, _c.c_int, _vp, _vp]),
-    "mgemv_probe_gemv": (_c.c_int, [_c.c_int, _vp, _vp, _u16p, _u16p, _u16p, _u16p, _c.c_int, _c.c_int, _c.c_int, _vp]),
+    "mgemv_probe_gemv": (_c.c_int, [_c.c_int, _vp, _c.c_size_t, _vp, _u16p, _u16p, _u16p, _u16p, _c.c_int, _c.c_int, _c.c_int, _vp]),
     "mgemv_probe_gemv_rows": (_c.c_int, [_c.c_int, _c.c_int, _vp, _u16p, _u16p, _u16p, _u16p, _c.c_int, _c.c_int, _c.c_int,
                                          _vp]),
     "mgemv_host_gemv": (_c.c_int, [_c.c_int] * 5 + [_vp] * 6 + [_c.c_int] * 2),

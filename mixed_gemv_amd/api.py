@@ -370,6 +370,7 @@ def probe_gemv_rows(kind, N, ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_D, M, 
 PROBE_LOADS_ONLY = 1
 PROBE_TIMELINE = 2
 PROBE_COMPUTE_ONLY = 3
+PROBE_TIMELINE_WAITS = 4
 
 
 def probe_empty_launch(stream=None):
@@ -390,10 +391,15 @@ def probe_stream_read(src, nbytes, workgroups, waves_per_workgroup, units_in_fli
                "probe_stream_read")
 
 
+PROBE_TIMELINE_WORDS = 14
+
+
 def probe_gemv(kind, trace, ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_D, M, K, group_size, stream=None):
     """Measurement builds of the headline kernel (mgemv_probe_gemv): PROBE_LOADS_ONLY, PROBE_COMPUTE_ONLY or PROBE_TIMELINE
-    (trace: int64 device tensor of 5 entries per wave)."""
-    _lib.check(_lib.lib().mgemv_probe_gemv(int(kind), _dev_ptr(trace), _dev_ptr(ptr_A), _dev_ptr(ptr_B),
+    (trace: int64 device tensor of PROBE_TIMELINE_WORDS entries per wave; its size is passed on as the capacity, and a
+    launch of more waves than it holds is refused)."""
+    capacity = 0 if trace is None else int(trace.numel()) // PROBE_TIMELINE_WORDS
+    _lib.check(_lib.lib().mgemv_probe_gemv(int(kind), _dev_ptr(trace), capacity, _dev_ptr(ptr_A), _dev_ptr(ptr_B),
                                            _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_D), int(M), int(K),
                                            int(group_size), _stream_ptr(stream)), "probe_gemv")
 

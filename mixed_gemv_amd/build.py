@@ -12,6 +12,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")   # objects and the compiler's intermediate files (the device assembly among them)
 LIB_PATH = os.path.join(LIB_DIR, "libmixed_gemv_amd.so")
 LINT_REPORT = os.path.join(LIB_DIR, "isa_lint.json")
+MIN_DOT_INSTRUCTIONS = 10000
 
 # One translation unit per family of kernel instantiations, so that they compile side by side.
 SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "gemv_kernels.hip", "probes.hip",
@@ -44,6 +45,9 @@ def lint_device_code(verbose=True):
     import json
     from . import isa_lint
     files = sorted(glob.glob(os.path.join(OBJ_DIR, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+    if not files:
+        raise RuntimeError(f"isa_lint: no device assembly (*-hip-amdgcn-amd-amdhsa-gfx950.s) under {OBJ_DIR}: "
+                           "the compiled kernels cannot be checked")
     reports = [isa_lint.lint_file(f) for f in files]
     with open(LINT_REPORT, "w") as f:
         json.dump(reports, f, indent=1)
@@ -53,6 +57,10 @@ def lint_device_code(verbose=True):
               f"{sum(r['kernels_with_dots'] for r in reports)} kernels of {len(files)} files, {bad} findings", flush=True)
     if bad:
         raise RuntimeError(f"isa_lint: {bad} hazards in the compiled kernels, see {LINT_REPORT}")
+    # the VALU kernels alone hold tens of thousands of dot instructions: a check that saw (almost) none checked nothing
+    if sum(r["dot_instructions"] for r in reports) < MIN_DOT_INSTRUCTIONS:
+        raise RuntimeError(f"isa_lint: only {sum(r['dot_instructions'] for r in reports)} dot instructions found in "
+                           f"{len(files)} files; the check did not see the kernels")
     return reports
 
 

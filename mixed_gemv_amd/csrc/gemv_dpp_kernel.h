@@ -319,6 +319,34 @@ __device__ __forceinline__ void finish_tile(float (&acc)[MB], float* slot) {
   }
 }
 
+// Timeline probe: what a wave's unit loop waits for.  Before a unit's arithmetic starts, the wave
+// stands in an explicit wait for that unit's operands and first weight block (everything requested
+// behind them -- the unit's other three blocks and the whole next unit -- may still be on its way);
+// the time spent there is added up per third of the wave's units, the longest single wait is
+// kept, and the moments at which the second and last third begin are recorded.
+struct TimelineWaits {
+  uint32_t wait[3];   // ticks of the 100 MHz clock spent waiting, per third of the wave's units
+  uint32_t longest;   // the longest single wait
+  uint64_t begin[2];  // when the second / last third of the units began
+};
+
+// kLoadsBehindFirstBlock: loads issued after block 0 of the unit that is about to be computed.
+template <int kLoadsBehindFirstBlock>
+__device__ __forceinline__ void timeline_wait(TimelineWaits& t, int u, int total) {
+  static_assert(kLoadsBehindFirstBlock >= 3 && kLoadsBehindFirstBlock < 64, "the counter of outstanding loads has 6 bits");
+  uint64_t a, b;
+  asm volatile("s_memrealtime %0\n\ts_waitcnt vmcnt(%2)\n\ts_memrealtime %1\n\ts_waitcnt lgkmcnt(0)"
+               : "=&s"(a), "=&s"(b) : "n"(kLoadsBehindFirstBlock) : "memory");
+  const uint32_t d = (uint32_t)(b - a);
+  const int third = u * 3 / total;
+  t.wait[0] += third == 0 ? d : 0u;
+  t.wait[1] += third == 1 ? d : 0u;
+  t.wait[2] += third == 2 ? d : 0u;
+  t.longest = d > t.longest ? d : t.longest;
+  if (third >= 1 && t.begin[0] == 0) t.begin[0] = a;
+  if (third >= 2 && t.begin[1] == 0) t.begin[1] = a;
+}
+
 // blockDim = (64 * split_k, tiles_per_wg).  Dynamic LDS: ceil(tiles / sequences) * tiles_per_wg *
 // split_k * MB * 64 floats.
 // One activation row, one group per run: ask for 6 resident waves per SIMD (at most 80 VGPRs).
@@ -329,7 +357,7 @@ __device__ __forceinline__ void finish_tile(float (&acc)[MB], float* slot) {
 // kProbeNone the product; kProbeComputeOnly loads a wave's first unit only and repeats its arithmetic
 // for every further unit; kProbeLoadsOnly keeps every load and replaces the arithmetic of a unit
 // by an exclusive-or over its registers -- what the access pattern alone takes; kProbeTimeline
-// records five timestamps per wave.
+// records timestamps and the time spent waiting for loads, per wave.
 template <int BITS, int QOP, int MB, int GROUPS_PER_RUN, bool MULTI, int ACT, int PROBE = kProbeNone>
 __global__ void __launch_bounds__(kWave * (MB >= 3 || ACT == kActBf16 ? kMaxWavesPerWideWorkgroup : kMaxWavesPerWorkgroup))
 __attribute__((amdgpu_waves_per_eu(ACT == kActF16 && MB == 1 && GROUPS_PER_RUN == 1 ? 6 : 1)))
@@ -337,7 +365,13 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
                 uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group, GemvTail tail) {
   extern __shared__ float partials[];
   uint64_t stamp[5] = {0, 0, 0, 0, 0};
-  if constexpr (PROBE == kProbeTimeline) stamp[0] = __builtin_amdgcn_s_memrealtime();
+  TimelineWaits waits{};
+  int units_computed = 0;
+  uint64_t cycles_at_start = 0;
+  if constexpr (PROBE == kProbeTimeline) {
+    stamp[0] = __builtin_amdgcn_s_memrealtime();
+    cycles_at_start = __builtin_readcyclecounter();
+  }
   Problem p;
   p.weights = weights;
   p.x = x;
@@ -458,6 +492,10 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         else load_unit<BITS, QOP, MB, GROUPS_PER_RUN>(fb, p, w_rsrc, x_rsrc, tables, cur);
         if (single_stage) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);  // keep the prefetch ahead of the arithmetic it overlaps
+        if constexpr (PROBE == kProbeTimeline) {
+          if (late.flags & kTimelineWaits) timeline_wait<kBlocksPerUnit - 1 + MB + GROUPS_PER_RUN * 2 + kBlocksPerUnit>(waits, u, total);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fa, c, short_ok);
         if constexpr (MULTI) {
           if (--pending == 0) {
@@ -472,6 +510,10 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
         if (single_stage) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         if (u + 1 < total) {
+          if constexpr (PROBE == kProbeTimeline) {
+            if (late.flags & kTimelineWaits) timeline_wait<kBlocksPerUnit - 1 + MB + GROUPS_PER_RUN * 2 + kBlocksPerUnit>(waits, u + 1, total);
+            __builtin_amdgcn_sched_barrier(0);
+          }
           compute_unit<BITS, QOP, MB, GROUPS_PER_RUN, ACT, PROBE>(acc, fb, c, short_ok);
           if constexpr (MULTI) {
             if (--pending == 0) {
@@ -488,6 +530,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
       __builtin_amdgcn_sched_barrier(0);
       asm volatile("" :: "v"(acc[0]));
       stamp[3] = __builtin_amdgcn_s_memrealtime();      // the last unit is computed
+      units_computed = total;
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (!MULTI) finish_tile<MB>(acc, partials + (ty * late.split_k + kw) * MB * kWave + lane_after_loop());
@@ -522,9 +565,16 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");    // the outputs are on their way
     stamp[4] = __builtin_amdgcn_s_memrealtime();
     if (late.trace != nullptr && lane_c == 0) {
-      unsigned long long* out = late.trace + ((size_t)blockIdx.x * (blockDim.x * blockDim.y / kWave) + ty * split_k + kw) * 5;
+      unsigned long long* out =
+          late.trace + ((size_t)blockIdx.x * (blockDim.x * blockDim.y / kWave) + ty * split_k + kw) * kTimelineWordsPerWave;
 #pragma unroll
       for (int i = 0; i < 5; ++i) out[i] = stamp[i];
+      out[5] = waits.wait[0]; out[6] = waits.wait[1]; out[7] = waits.wait[2];
+      out[8] = waits.longest;
+      out[9] = waits.begin[0]; out[10] = waits.begin[1];
+      out[11] = (unsigned long long)units_computed;
+      out[12] = cycles_at_start;
+      out[13] = __builtin_readcyclecounter();
     }
   }
 }

@@ -561,7 +561,8 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
              const uint16_t* bias, uint16_t* y, int batch_count, int n_out, int m_batch, int k, int group_size,
              int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
              int64_t stride_bias, int64_t stride_y, void* stream, int act, float alpha = 1.0f, float beta = 1.0f,
-             int probe = kProbeNone, unsigned long long* trace = nullptr) {
+             int probe = kProbeNone, unsigned long long* trace = nullptr, size_t trace_capacity_waves = 0,
+             bool timed_waits = false) {
   if (batch_count < 1 || batch_count > 65535) return MGEMV_ERR_BATCH;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
@@ -588,7 +589,7 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
   g.tail.bias = reinterpret_cast<const half_t*>(bias);
   g.tail.split_k = g.plan.split_k;
   g.tail.num_groups = k / group_size;
-  g.tail.flags = g_dequant_flags.load() | (g.plan.stages == 1 ? kSingleStage : 0);
+  g.tail.flags = g_dequant_flags.load() | (g.plan.stages == 1 ? kSingleStage : 0) | (timed_waits ? kTimelineWaits : 0);
   g.tail.alpha = alpha;
   g.tail.beta = beta;
   g.tail.trace = trace;
@@ -633,6 +634,10 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
     g.x = reinterpret_cast<const half_t*>(x);
     g.tail.y = reinterpret_cast<half_t*>(y);
     g.lds = (size_t)g.plan.tiles_in_sequence * g.plan.tiles_per_wg * g.plan.split_k * kWave * sizeof(float);
+    // every launched wave writes its own row of the trace: the caller's buffer must hold them all
+    if (probe == kProbeTimeline &&
+        (size_t)g.grid.x * (size_t)(g.plan.split_k * g.plan.tiles_per_wg) > trace_capacity_waves)
+      return MGEMV_ERR_SIZE;
     return launch_gemv_probe(g, probe) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
   }
   // VALU path: activation rows are processed kMaxValuBatch at a time.
@@ -727,7 +732,7 @@ namespace {
 int probe_kind(int kind) {
   return kind == MGEMV_PROBE_LOADS_ONLY     ? mgemv::kProbeLoadsOnly
          : kind == MGEMV_PROBE_COMPUTE_ONLY ? mgemv::kProbeComputeOnly
-                                            : mgemv::kProbeTimeline;
+                                            : mgemv::kProbeTimeline;   // with or without the per-unit waits
 }
 }  // namespace
 
@@ -739,13 +744,16 @@ int mgemv_probe_gemv_rows(int kind, int m_batch, const void* weights, const uint
                          probe_kind(kind), nullptr);
 }
 
-int mgemv_probe_gemv(int kind, unsigned long long* trace, const void* weights, const uint16_t* x, const uint16_t* scale,
-                     const uint16_t* zero_add, uint16_t* y, int n_out, int k, int group_size, void* stream) {
-  if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_TIMELINE && kind != MGEMV_PROBE_COMPUTE_ONLY) return MGEMV_ERR_SIZE;
-  if (kind == MGEMV_PROBE_TIMELINE && (trace == nullptr || reinterpret_cast<uintptr_t>(trace) % 8)) return MGEMV_ERR_NULL_POINTER;
+int mgemv_probe_gemv(int kind, unsigned long long* trace, size_t trace_capacity_waves, const void* weights,
+                     const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add, uint16_t* y, int n_out, int k,
+                     int group_size, void* stream) {
+  if (kind != MGEMV_PROBE_LOADS_ONLY && kind != MGEMV_PROBE_TIMELINE && kind != MGEMV_PROBE_COMPUTE_ONLY &&
+      kind != MGEMV_PROBE_TIMELINE_WAITS)
+    return MGEMV_ERR_SIZE;
+  if ((kind == MGEMV_PROBE_TIMELINE || kind == MGEMV_PROBE_TIMELINE_WAITS) && (trace == nullptr || reinterpret_cast<uintptr_t>(trace) % 8)) return MGEMV_ERR_NULL_POINTER;
   return mgemv::gemv_any(weights, x, scale, zero_add, nullptr, y, 1, n_out, 1, k, group_size,
                          MGEMV_FINEGRAINED_SCALE_AND_ZEROS, 4, 0, 0, 0, 0, 0, stream, mgemv::kActF16, 1.0f, 1.0f,
-                         probe_kind(kind), trace);
+                         probe_kind(kind), trace, trace_capacity_waves, kind == MGEMV_PROBE_TIMELINE_WAITS);
 }
 
 // gemv/device/gemv_adaptor.h:114-178 as one plain struct.

@@ -7,6 +7,7 @@
 
 #include "device_math.h"
 #include "mixed_gemv.h"
+#include "mixed_gemv_probes.h"
 #include "tile_layout.h"
 
 namespace mgemv {
@@ -20,6 +21,8 @@ constexpr int kNumCus = 256;
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
 constexpr int kSingleStage = 2;           // GemvTail::flags: no load in flight while a unit is computed (VALU kernel)
+constexpr int kTimelineWaits = 8;         // GemvTail::flags, timeline probe: time the wait in front of every unit as well
+constexpr int kTimelineWordsPerWave = MGEMV_PROBE_TIMELINE_WORDS;  // 64-bit words the timeline probe writes per wave
 constexpr int kProbeNone = 0, kProbeLoadsOnly = 1, kProbeTimeline = 2, kProbeComputeOnly = 3;  // measurement builds of the VALU kernel
 
 // Kernel arguments.  The first ten (four pointers and six 32-bit words, 14 dwords) are what a
@@ -36,7 +39,7 @@ struct GemvTail {
   int seq_base;        // VALU kernel: tiles / sequences ...
   int seq_rem;         // ... and tiles % sequences (the first seq_rem sequences get one tile more)
   long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
-  unsigned long long* trace;  // timeline probe: five timestamps per wave, else unused
+  unsigned long long* trace;  // timeline probe: kTimelineWordsPerWave words per wave, else unused
 };
 
 // Scalar view of one problem inside a kernel.

@@ -195,7 +195,37 @@ class GemvAdaptor {
     run(stream);
   }
 
+  // gemv/device/gemv_adaptor.h:190-196 (get_grid_size / get_block_size of Params).  The reference's
+  // launch shape is a compile-time function of the problem's rows (ceil(M / 64) blocks of 128
+  // threads); here it is the launch plan of the problem (mgemv_query_launch_for: built-in rules,
+  // tuned plans, overrides), so both take the arguments and, since the plan is made for the
+  // compute units of the device the launch goes to, that count (256: an unpartitioned MI355X).
+  struct Dim3 {
+    unsigned x, y, z;
+  };
+  Dim3 get_grid_size(const Arguments& args, int num_compute_units = 256) const {
+    const LaunchShape s = launch_shape(args, num_compute_units);
+    return Dim3{(unsigned)((s.workgroups + 7) / 8 * 8), 1u, (unsigned)args.batch_count};  // whole rounds over the 8 XCDs
+  }
+  Dim3 get_block_size(const Arguments& args, int num_compute_units = 256) const {
+    const LaunchShape s = launch_shape(args, num_compute_units);
+    return Dim3{(unsigned)(64 * s.k_split_waves), (unsigned)s.tiles_per_workgroup, 1u};
+  }
+
  private:
+  struct LaunchShape {
+    int workgroups, k_split_waves, tiles_per_workgroup;
+  };
+  LaunchShape launch_shape(const Arguments& a, int num_compute_units) const {
+    int out[12] = {0};
+    const int group = quant_op_ == WeightOnlyQuantOp::PER_COLUMN_SCALE_ONLY ? a.problem_size.k() : a.group_size;
+    check(mgemv_query_launch_for(a.problem_size.m(), a.problem_size.n(), a.problem_size.k(), weight_bits_, group,
+                                 element_ == ElementType::kBFloat16 ? MGEMV_ELEMENT_BF16 : MGEMV_ELEMENT_F16,
+                                 num_compute_units, out),
+          "GemvAdaptor::get_grid_size");
+    return LaunchShape{out[0], out[2], out[3]};
+  }
+
   WeightOnlyQuantOp quant_op_;
   int weight_bits_;
   ElementType element_;

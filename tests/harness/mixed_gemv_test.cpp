@@ -97,6 +97,22 @@ int main(int argc, char** argv) {
   HIP_CHECK(hipMemcpy(d_bias, h_bias.data(), h_bias.size() * 2, hipMemcpyHostToDevice));
   HIP_CHECK(hipMemset(d_D, 0xff, (size_t)B * M * kGemmN * 2));
 
+  {
+    // the launch shape, under the reference's names (gemv/device/gemv_adaptor.h:190-196)
+    GemvAdaptor::Arguments shape_args;
+    shape_args.problem_size = GemmCoord{M, kGemmN, K};
+    shape_args.group_size = group_size;
+    shape_args.batch_count = B;
+    GemvAdaptor op(quant_op, bits);
+    const GemvAdaptor::Dim3 grid = op.get_grid_size(shape_args), block = op.get_block_size(shape_args);
+    std::printf("grid (%u, %u, %u) block (%u, %u, %u)\n", grid.x, grid.y, grid.z, block.x, block.y, block.z);
+    if (grid.x == 0 || grid.x % 8 != 0 || grid.y != 1 || grid.z != (unsigned)B || block.x % 64 != 0 || block.x == 0 ||
+        block.y == 0 || block.x * block.y > 1024 || block.z != 1) {
+      std::printf("implausible launch shape\n");
+      return 6;
+    }
+  }
+
   try {
     for (int i = 0; i < 20; i++)
       device_gemv(d_A, d_B, d_scale, d_zero_point, with_bias ? d_bias : nullptr, d_D, B, M, kGemmN, K, group_size, quant_op, bits);

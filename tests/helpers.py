@@ -143,3 +143,28 @@ class DeviceProblem:
         torch.cuda.synchronize()
         out = out.cpu().numpy()
         return out.view(np.uint16) if p.element == "bf16" else out.view(np.float16)
+
+
+def float64_bound_violations(prob, y, rows_per_chunk=2048, dq=None):
+    """How many outputs lie outside what the mathematics allows ANY correct kernel: with the
+    (bit-exact) dequantised weights dq, the exactly accumulated sum  x . dq[n] + bias[n]  in float64,
+    and around it the classical bound for k products (exact in fp32) summed in fp32 in any order,
+    k * 2^-24 * sum |x| |dq|, plus one rounding to fp16 (2^-11 relative, 2^-24 absolute for
+    subnormal results).  Unlike a relative error against HOST_CHECK this needs no floor: outputs
+    that cancel to almost zero are bounded by the magnitude of what cancelled.
+    dq: the oracle's dequantised weights if the caller already has them.
+    Returns (violations, largest error / bound)."""
+    dq = prob.oracle_dequant() if dq is None else dq
+    x = prob.x.astype(np.float64)
+    y = np.asarray(y).astype(np.float64).reshape(prob.m_batch, prob.n_out)
+    bias = prob.bias.astype(np.float64) if prob.bias is not None else np.zeros(prob.n_out)
+    bad, worst = 0, 0.0
+    for r0 in range(0, prob.n_out, rows_per_chunk):
+        d = dq[r0:r0 + rows_per_chunk].astype(np.float64)
+        exact = x @ d.T + bias[None, r0:r0 + rows_per_chunk]
+        mag = np.abs(x) @ np.abs(d.T) + np.abs(bias[None, r0:r0 + rows_per_chunk])
+        bound = mag * (prob.k + 1) * 2.0 ** -24 + np.abs(exact) * 2.0 ** -11 + 2.0 ** -24
+        err = np.abs(y[:, r0:r0 + rows_per_chunk] - exact)
+        bad += int((err > bound).sum())
+        worst = max(worst, float((err / bound).max()))
+    return bad, worst

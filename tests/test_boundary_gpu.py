@@ -147,6 +147,26 @@ def test_reduction_length_a_multiple_of_8_only(gpu, bits, k, m_batch):
     assert rel <= REL_TOL
 
 
+@pytest.mark.parametrize("bits,k", [(4, 4104), (4, 520), (4, 8), (8, 264)])
+@pytest.mark.parametrize("m_batch", [5, 8, 16])
+def test_reduction_length_a_multiple_of_8_only_register_operand_kernel(gpu, bits, k, m_batch):
+    """The same through the register-operand matrix-core kernel, which loads its activation operand
+    in 8-element pieces of its own: a single tile (the only shape that kernel serves by itself),
+    and a larger matrix with the kernel forced."""
+    for n_out, force in ((16, False), (96, True)):
+        prob = Problem(f"k8r_{bits}_{k}", n_out, k, bits, PER_COLUMN, 0, m_batch=m_batch, bias=True, x_dist="normal")
+        dev = DeviceProblem(prob, gpu)
+        try:
+            if force:
+                mg.set_matrix_core_variant(mg.MATRIX_CORE_REGISTER_OPERAND)
+            assert mg.query_launch(n_out, m_batch, k, bits)["matrix_core"] == 1
+            y = dev.run()
+        finally:
+            mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
+        _, rel, _ = error_report(y, prob.oracle_gemv(threads=8))
+        assert rel <= REL_TOL, (n_out, rel)
+
+
 @pytest.mark.parametrize("bits,qop,g", [(4, SCALE_AND_ZEROS, 128), (8, PER_COLUMN, 0)])
 def test_weights_preprocessed_from_row_major_input(gpu, bits, qop, g):
     """utils/preprocess.h:507-511: a [k][n_out] row-major matrix is transposed first.  The buffer the

@@ -111,6 +111,48 @@ def test_one_hot_activation_is_bit_exact_through_the_gemv_kernel(gpu):
         assert np.all((y[~nz] & 0x7FFF) == 0), j
 
 
+@pytest.mark.parametrize("split,tw", [(0, 1), (4, 1), (2, 2), (2, 4), (1, 8)])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_one_hot_rows_are_bit_exact_through_the_matrix_core_kernel(gpu, bits, split, tw):
+    """One-hot activation rows, each at a k of its own, through v_mfma_f32_16x16x32_bf16: y[b][n] == dq[n][k_b]
+    bit for bit (up to the sign of a zero), with a stage per wave and with stages shared by 2, 4 and 8 tiles,
+    8 and 16 staged rows, the fused and the general dequantiser."""
+    import torch
+    k = 1536 if bits == 4 else 768
+    for m_batch, scale_range in ((5, (1e-4, 0.02)), (8, (1e-4, 0.02)), (16, (1e-4, 0.02)), (13, (1e-4, 0.02))):
+        if (8 if m_batch <= 8 else 16) // tw < 2:
+            continue
+        prob = Problem(f"b_mc_onehot{bits}", 112, k, bits, SCALE_AND_ZEROS, 64, m_batch=m_batch, scale_range=scale_range,
+                       element="bf16")
+        if m_batch == 13:      # scales outside the fused form's range (negative, tiny): the general dequantiser
+            prob.scale[::2, ::3] = 0xBC80
+            prob.scale[1::2, 1::3] = 0x0C00
+        dq = prob.oracle_dequant()
+        dev = DeviceProblem(prob, gpu)
+        try:
+            mg.set_matrix_core_threshold(1)
+            mg.set_launch_override(split, tw, 0, 0)
+            plan = mg.query_launch(prob.n_out, m_batch, k, bits, element="bf16")
+            assert plan["matrix_core"] == 2 and plan["tiles_per_wg"] == tw, plan
+            for trial in range(4):
+                hot = [(b * 37 + trial * 131) % k for b in range(m_batch)]
+                if trial == 0:
+                    hot[:4] = [0, k - 1, 511 if bits == 4 else 255, 512 if bits == 4 else 256][:m_batch]
+                x = np.zeros((m_batch, k), dtype=np.uint16)
+                x[np.arange(m_batch), hot] = 0x3F80
+                dev.x = torch.from_numpy(x.view(np.int16)).to(gpu)
+                got = dev.run()
+                for b in range(m_batch):
+                    want = dq[:, hot[b]]
+                    finite = (want & 0x7F80) != 0x7F80
+                    nz = ((want & 0x7FFF) != 0) & finite
+                    assert np.array_equal(got[b][nz], want[nz]), (m_batch, trial, b, hot[b])
+                    assert np.all((got[b][~nz & finite] & 0x7FFF) == 0)
+        finally:
+            mg.set_matrix_core_threshold(0)
+            mg.set_launch_override(0, 0, 0, 0)
+
+
 def test_split_k_and_tile_walk_invariance(gpu):
     prob = Problem("b_splitk", 192, 8192, 4, SCALE_AND_ZEROS, 128, bias=True, x_dist="normal", element="bf16")
     dev = DeviceProblem(prob, gpu)

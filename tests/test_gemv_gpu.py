@@ -8,7 +8,8 @@ import pytest
 
 import mixed_gemv_amd as mg
 import oracle as orc
-from helpers import PER_COLUMN, SCALE_AND_ZEROS, SCALE_ONLY, DeviceProblem, Problem, error_report
+from helpers import (PER_COLUMN, SCALE_AND_ZEROS, SCALE_ONLY, DeviceProblem, Problem, error_report,
+                     float64_bound_violations)
 
 pytestmark = pytest.mark.gpu
 
@@ -206,6 +207,59 @@ def test_one_hot_activation_is_bit_exact_through_the_gemv_kernel(gpu):
             nz = (want & 0x7FFF) != 0
             assert np.array_equal(got[nz], want[nz]), (bits, kk)
             assert np.all((got[~nz] & 0x7FFF) == 0)
+
+
+# (matrix-core variant, k-split waves, tiles per workgroup): the LDS-staged kernel with a stage per wave
+# (one tile per workgroup) and with stages shared by 2, 4 and 8 tiles, and the register-operand kernel
+MATRIX_CORE_LAUNCHES = [("lds_own_stages", "lds", 0, 1), ("lds_own_stages_split4", "lds", 4, 1), ("lds_shared_by_2", "lds", 2, 2),
+                        ("lds_shared_by_4", "lds", 2, 4), ("lds_shared_by_8", "lds", 1, 8), ("register_operand", "reg", 0, 0)]
+
+
+@pytest.mark.parametrize("launch", MATRIX_CORE_LAUNCHES, ids=[c[0] for c in MATRIX_CORE_LAUNCHES])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_one_hot_rows_are_bit_exact_through_the_matrix_core_kernels(gpu, bits, launch):
+    """Every activation row is a one-hot vector at a k of its own: y[b][n] == dq[n][k_b] bit for bit (up
+    to the sign of a zero) through v_mfma_f32_16x16x32_f16 -- a product with 1 and sums with zeros are
+    exact in the matrix core too.  Pins the dequantiser inside both matrix-core kernels and which
+    lane's weights meet which activation (the LDS stage's layout, 8 and 16 staged rows, shared and
+    own stages, the register operand's loads), which a tolerance against the VALU kernel does not."""
+    import torch
+    _, variant, split, tw = launch
+    k = 1536 if bits == 4 else 768
+    rng = np.random.default_rng(bits * 100 + split * 10 + tw)
+    for m_batch, scale_range in ((5, (1e-4, 0.02)), (8, (0.02, 0.3)), (16, (1e-4, 0.02)), (13, (0.02, 0.3))):
+        if variant == "lds" and tw and (8 if m_batch <= 8 else 16) // tw < 2:
+            continue    # that many tiles cannot share a stage of 8 rows
+        prob = Problem(f"mc_onehot{bits}", 112, k, bits, SCALE_AND_ZEROS, 64, m_batch=m_batch, scale_range=scale_range)
+        dev = DeviceProblem(prob, gpu)
+        dq = prob.oracle_dequant().view(np.uint16)
+        try:
+            mg.set_matrix_core_threshold(1)
+            mg.set_matrix_core_variant(mg.MATRIX_CORE_LDS_STAGED if variant == "lds" else mg.MATRIX_CORE_REGISTER_OPERAND)
+            mg.set_launch_override(split, tw, 0, 0)
+            plan = mg.query_launch(prob.n_out, m_batch, k, bits)
+            assert plan["matrix_core"] == (2 if variant == "lds" else 1), plan
+            if variant == "lds" and tw:
+                assert plan["tiles_per_wg"] == tw, plan
+            for trial in range(6):
+                # first trials: k positions that exercise every lane group, block and word of a unit
+                hot = ([(b * 37 + trial * 131) % k for b in range(m_batch)] if trial < 4
+                       else list(rng.integers(0, k, m_batch)))
+                if trial == 0:
+                    hot[:4] = [0, k - 1, 511 if bits == 4 else 255, 512 if bits == 4 else 256][:m_batch]
+                x = np.zeros((m_batch, k), dtype=np.float16)
+                x[np.arange(m_batch), hot] = 1.0
+                dev.x.copy_(torch.from_numpy(x.view(np.int16)))
+                got = dev.run().view(np.uint16)
+                for b in range(m_batch):
+                    want = dq[:, hot[b]]
+                    nz = (want & 0x7FFF) != 0
+                    assert np.array_equal(got[b][nz], want[nz]), (m_batch, trial, b, hot[b])
+                    assert np.all((got[b][~nz] & 0x7FFF) == 0)
+        finally:
+            mg.set_matrix_core_threshold(0)
+            mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
+            mg.set_launch_override(0, 0, 0, 0)
 
 
 def test_bias_only_and_output_fully_written(gpu):
@@ -590,9 +644,9 @@ def test_hip_graph_replays_match_eager_launches(gpu):
 
 
 def test_reference_shipped_shape(gpu):
-    """The shape the reference's main() ships with (mixed_gemv_test.cu:187-191), reduced 4x along
-    the vocabulary dimension to keep the CPU side short: out = 37984, K = 2048, int4 g128 scale+zero."""
-    prob = Problem("ref_main", 37984, 2048, 4, SCALE_AND_ZEROS, 128, scale_range=(0.1, 0.3), zero_kind="int8")
+    """The problem the reference's main() ships with (mixed_gemv_test.cu:187-191) at full size:
+    out = 151936, K = 2048, int4 g128 scale+zero, its own scale range and int8 zero points."""
+    prob = Problem("ref_main", 151936, 2048, 4, SCALE_AND_ZEROS, 128, scale_range=(0.1, 0.3), zero_kind="int8")
     dev, y = check(prob, gpu, dequant=False)
     ref = prob.oracle_gemv(threads=16)
     abs_err = np.abs(y.astype(np.float64) - ref.astype(np.float64))
@@ -603,3 +657,37 @@ def test_reference_shipped_shape(gpu):
     _, _, floor = error_report(y, ref)
     ulp = np.spacing(np.maximum(np.abs(ref), floor).astype(np.float16)).astype(np.float64)
     assert np.all(abs_err <= 2 * ulp)
+    bad, worst = float64_bound_violations(prob, y, rows_per_chunk=8192)
+    assert bad == 0, (bad, worst)
+
+
+# tag, n_out, k, group, activation rows run (each on the first rows of one set of activations), bias, x
+BOUND_CASES = [
+    ("c5", 28672, 8192, 128, (1,), False, "normal"),
+    ("c4", 8192, 8192, 64, (1, 2, 4, 8, 16), True, "uniform"),
+    ("vocab", 128256, 4096, 128, (1,), False, "normal"),
+]
+
+
+@pytest.mark.parametrize("cfg", BOUND_CASES, ids=[c[0] for c in BOUND_CASES])
+def test_full_size_outputs_within_the_float64_bound(gpu, cfg):
+    """At BASELINE's full sizes, every output of the kernel -- VALU at 1-2 rows, matrix cores from 4 --
+    lies within the fp32-accumulation bound around the exactly accumulated sum of the dequantised
+    weights (helpers.float64_bound_violations): the property the oracle's own HOST_CHECK loop is held
+    to (test_oracle_gemv.py), which needs no denominator floor."""
+    tag, n_out, k, g, rows, bias, xd = cfg
+    prob = Problem(tag + "_bound", n_out, k, 4, SCALE_AND_ZEROS, g, m_batch=max(rows), bias=bias, x_dist=xd)
+    dev = DeviceProblem(prob, gpu)
+    full_x, full_rows = prob.x, prob.m_batch
+    dq = prob.oracle_dequant()
+    for m in rows:
+        prob.m_batch, prob.x = m, full_x[:m]
+        dev.y.fill_(0x7e00)
+        mg.device_gemv(dev.w, dev.x, dev.scale, dev.zero, dev.bias, dev.y, 1, n_out, m, k, g, SCALE_AND_ZEROS, 4)
+        import torch
+        torch.cuda.synchronize()
+        y = dev.y.cpu().numpy().view(np.float16)[:m]
+        bad, worst = float64_bound_violations(prob, y, dq=dq)
+        print(f"{tag} M={m}: largest error / bound = {worst:.3f}", flush=True)
+        assert bad == 0, (m, bad, worst)
+    prob.m_batch, prob.x = full_rows, full_x

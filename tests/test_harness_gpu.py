@@ -10,6 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 BINARY = os.path.join(HERE, "harness", "mixed_gemv_test")
 
 CASES = [
+    ["151936", "2048", "128", "3", "4", "0"],  # the problem the reference's main() ships with (mixed_gemv_test.cu:187), at full size
     ["11008", "2048", "128", "3", "4", "0"],   # one of the reference's own shapes (mixed_gemv_test.cu:189), mode as shipped
     ["2048", "11008", "128", "3", "4", "1"],   # the other one (:188), with the bias epilogue
     ["4096", "4096", "128", "2", "4", "1"],

@@ -21,12 +21,15 @@ COL, ROW = mg.LayoutType.kColumnMajor, mg.LayoutType.kRowMajor
 INT4_FIELD_SHIFT = (7, 23, 3, 19, 15, 31, 11, 27)
 
 def test_library_exports_every_declared_symbol():
-    header = open(os.path.join(REPO, "include", "mixed_gemv.h")).read()
+    # the boundary (mixed_gemv.h) and the measurement probes (mixed_gemv_probes.h) are one library
+    header = "".join(open(os.path.join(REPO, "include", h)).read() for h in ("mixed_gemv.h", "mixed_gemv_probes.h"))
     declared = set(re.findall(r"MGEMV_API\s+[\w\s\*]+?\b(mgemv_\w+)\s*\(", header))
     assert len(declared) >= 12
+    boundary = open(os.path.join(REPO, "include", "mixed_gemv.h")).read()
+    assert "mgemv_probe_" not in boundary, "measurement entries belong in mixed_gemv_probes.h"
     handle = ctypes.CDLL(_lib.LIB_PATH)
     for name in declared:
-        assert hasattr(handle, name), f"{name} declared in include/mixed_gemv.h but not exported"
+        assert hasattr(handle, name), f"{name} declared in include/ but not exported"
     assert declared == set(_lib.SIGNATURES), "python binding and header disagree"
     assert _lib.lib().mgemv_version() >= 100
     for code in range(0, 17):

@@ -1,4 +1,4 @@
-"""The measurement probes of the library (include/mixed_gemv.h, "Measurement probes"): they run,
+"""The measurement probes of the library (include/mixed_gemv_probes.h): they run,
 the timeline build of the kernel still computes the GEMV, and its timestamps are ordered."""
 import numpy as np
 import pytest
@@ -18,9 +18,13 @@ def test_timeline_build_is_the_product_kernel_plus_timestamps(gpu, n_out, k, cap
     try:
         mg.set_launch_override(0, 0, 0, cap)
         want = dev.run().copy()
-        plan = mg.query_launch(n_out, 1, k, 4, 128)
-        waves = plan["workgroups"] * plan["threads"] // 64
-        trace = torch.zeros((waves, 5), dtype=torch.int64, device=gpu)
+        cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+        plan = mg.query_launch(n_out, 1, k, 4, 128, num_compute_units=cus)
+        waves = -(-plan["workgroups"] // 8) * 8 * plan["threads"] // 64      # the grid is a multiple of 8 workgroups
+        with pytest.raises(MixedGemvError):                                  # a trace that is too small is refused
+            mg.probe_gemv(mg.PROBE_TIMELINE, torch.zeros((waves - 1, mg.PROBE_TIMELINE_WORDS), dtype=torch.int64, device=gpu),
+                          dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 128)
+        trace = torch.zeros((waves, mg.PROBE_TIMELINE_WORDS), dtype=torch.int64, device=gpu)
         dev.y.fill_(0x7e00)
         mg.probe_gemv(mg.PROBE_TIMELINE, trace, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 128)
         torch.cuda.synchronize()
@@ -28,8 +32,15 @@ def test_timeline_build_is_the_product_kernel_plus_timestamps(gpu, n_out, k, cap
         t = trace.cpu().numpy()
         t = t[t[:, 0] > 0]                                  # workgroups past the last tile leave before stamping
         assert len(t) >= (n_out // 16) * plan["split_k"] // max(plan["tiles_in_sequence"], 1) // 2
-        assert np.all(np.diff(t, axis=1) >= 0)              # entry <= requested <= arrived <= computed <= stored
+        assert np.all(np.diff(t[:, :5], axis=1) >= 0)       # entry <= requested <= arrived <= computed <= stored
         assert (t[:, 4] - t[:, 0]).max() < 100_000          # 10 ns ticks: under a millisecond
+        units = plan["steps_per_wave"] * plan["tiles_in_sequence"]
+        assert t[:, 11].max() == units and t[:, 11].min() >= 0
+        loop = t[t[:, 11] >= 2]                              # waves of two or more units run the loop and time their waits
+        assert np.all(loop[:, 5:8].sum(axis=1) <= loop[:, 3] - loop[:, 1])   # waits lie inside the loop
+        assert np.all(loop[:, 8] <= loop[:, 5:8].sum(axis=1))
+        later = loop[loop[:, 9] > 0]
+        assert np.all((later[:, 9] >= later[:, 1]) & (later[:, 9] <= later[:, 3]))
         mg.probe_gemv(mg.PROBE_LOADS_ONLY, None, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 128)
         torch.cuda.synchronize()
     finally:
