@@ -197,6 +197,52 @@ def tune(n_out, k, weight_bits=4, quant_op=api.WeightOnlyQuantOp.FINEGRAINED_SCA
                 measurements=[(us, _describe(c)) for us, c, _ in results])
 
 
+def reconfirm(entry, device="cuda:0", launches=400, rounds=5, seed=1, cold_bytes=_CACHE_BYTES, quant_op=None, bias=False):
+    """Measures an existing table entry against the built-in plan once more, in alternation, on the
+    device at hand, and appends the gain in per cent (positive: the entry is ahead) to
+    entry["confirmations"].  A gain found on one machine at one time can be that machine's: boxes of
+    the same kind differ by several per cent among themselves (28672 x 8192: 22.4-24.4 us from lease
+    to lease), so an entry should only ship after `confirmed()` -- the gain shown again on another
+    lease.  Returns the gain.  Like tune(), must not run while other threads launch GEMVs."""
+    import statistics
+    import torch
+    device = torch.device(device)
+    element = entry.get("element", "f16")
+    per_column = entry["group_size"] == entry["k"]
+    qop = api.WeightOnlyQuantOp(quant_op) if quant_op is not None else (
+        api.WeightOnlyQuantOp.PER_COLUMN_SCALE_ONLY if per_column else api.WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS)
+    prob = _Problem(entry["n_out"], entry["k"], entry["weight_bits"], qop, entry["group_size"], entry["m_batch"], bias,
+                    device, seed, cold_bytes, element)
+    cand = {k: entry.get(k, 0) for k in ("kernel", "split_k", "tiles_per_wg", "tiles_per_wave", "max_workgroups")}
+    if entry.get("stages"):
+        cand["stages"] = entry["stages"]
+    builtin, tuned = [], []
+    try:
+        with torch.cuda.device(device):
+            _apply(dict(kernel=api.KERNEL_AUTO))
+            spin = time.perf_counter()
+            while time.perf_counter() - spin < 0.5:
+                prob.time_us(launches)
+            for _ in range(rounds):
+                _apply(dict(kernel=api.KERNEL_AUTO))
+                builtin.append(prob.time_us(launches))
+                _apply(cand)
+                tuned.append(prob.time_us(launches))
+    finally:
+        _apply(dict(kernel=api.KERNEL_AUTO))
+        api.set_prefetch_stages(0)
+    gain = round(100.0 * (statistics.median(builtin) / statistics.median(tuned) - 1.0), 2)
+    entry.setdefault("confirmations", []).append(gain)
+    return gain
+
+
+def confirmed(entry, min_gain=0.02, leases=2):
+    """True when the entry's gain over the built-in plan reached `min_gain` in at least `leases`
+    separate confirmation runs (reconfirm) and it was never behind by that much."""
+    gains = entry.get("confirmations", [])
+    return (sum(1 for g in gains if g >= 100.0 * min_gain) >= leases) and all(g > -100.0 * min_gain for g in gains)
+
+
 def _apply(cand):
     kernel = cand.get("kernel", api.KERNEL_AUTO)
     api.set_prefetch_stages(cand.get("stages", 2))  # 2 is the built-in value; any override set bypasses the table

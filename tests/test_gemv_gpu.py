@@ -348,6 +348,17 @@ def test_tuner_measures_installs_and_keeps_parity(gpu, m_batch):
         autotune.clear()
 
 
+def test_reconfirm_measures_an_entry_against_the_built_in_plan_and_leaves_no_override(gpu):
+    from mixed_gemv_amd import autotune
+    entry = dict(n_out=2048, k=4096, weight_bits=4, group_size=128, m_batch=1, element="f16", kernel=mg.KERNEL_VALU,
+                 split_k=1, tiles_per_wg=1, max_workgroups=8)     # a poor plan: 8 workgroups walk everything
+    before = mg.query_launch(2048, 1, 4096, 4, 128)
+    gain = autotune.reconfirm(entry, launches=64, rounds=2, cold_bytes=8 << 20)
+    assert entry["confirmations"] == [gain] and gain < -20.0, gain        # clearly behind the built-in plan
+    assert not autotune.confirmed(entry)
+    assert mg.query_launch(2048, 1, 4096, 4, 128) == before and mg.tuned_plan_count() == 0
+
+
 @pytest.mark.parametrize("tag,n_out,k,bits,qop,g,m_batch,cap", [
     ("st_ns", 4096, 4096, 4, SCALE_AND_ZEROS, 128, 1, 0),        # four waves of two units
     ("st_walk", 1024, 8192, 4, SCALE_AND_ZEROS, 128, 1, 8),      # walks of eight tiles

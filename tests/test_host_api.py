@@ -530,6 +530,9 @@ def test_default_plan_table_is_the_shipped_json_and_applies_to_256_compute_units
         if e.get("kernel"):
             assert got["matrix_core"] == kinds[e["kernel"]]
         assert e["us"] < e["builtin_us"] * 0.98
+        # ... and the gain was seen again on at least two separate leases, and the entry was never behind
+        from mixed_gemv_amd import autotune
+        assert autotune.confirmed(e), e.get("confirmations")
         # the entry covers the problem like any plan
         cov = mg.plan_coverage(*key, element=e["element"], num_compute_units=256)
         assert cov["tiles_miscovered"] == 0 and cov["bad_waves"] == 0
@@ -552,3 +555,13 @@ def _with_defaults_off(fn):
         return fn()
     finally:
         mg.set_default_plans(True)
+
+
+def test_an_entry_ships_only_after_two_confirmations():
+    from mixed_gemv_amd import autotune
+    assert not autotune.confirmed({})
+    assert not autotune.confirmed({"confirmations": [3.1]})
+    assert not autotune.confirmed({"confirmations": [3.1, 0.4, 1.9]})
+    assert autotune.confirmed({"confirmations": [3.1, 0.4, 2.0]})
+    assert not autotune.confirmed({"confirmations": [3.1, 2.4, -2.2]})      # behind once by as much as it gains
+    assert autotune.confirmed({"confirmations": [5.0, 4.0]}, min_gain=0.04) and not autotune.confirmed({"confirmations": [5.0, 4.0]}, leases=3)
