@@ -253,16 +253,25 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
  * from 3 rows on 1536 or more tiles; never for a single row); 17 keeps every batch size on the VALU kernel.  For tuning and tests.  Process-wide. */
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
-/* Which of the two matrix-core kernels serves the small batches:
+/* Which of the matrix-core kernels serves the small batches:
  *   MGEMV_MATRIX_CORE_AUTO (default)          the LDS-staged kernel wherever the matrix has at least two
  *                                             16-row tiles, else the register-operand kernel;
  *   MGEMV_MATRIX_CORE_REGISTER_OPERAND        always the kernel that reads its activation operand from
  *                                             L2 into registers;
  *   MGEMV_MATRIX_CORE_LDS_STAGED              the LDS-staged kernel wherever the matrix has at least two
- *                                             tiles.
+ *                                             tiles;
+ *   MGEMV_MATRIX_CORE_K_STATIONARY            the kernel whose waves each keep one k step of 512 (int4) or 256
+ *                                             (int8) reduction elements and its activation operand in registers
+ *                                             while the workgroup walks its tiles, wherever k has at most 16 such
+ *                                             steps (fp16 only; else as AUTO).
  * Same results to tolerance either way (the k split, hence the order of the fp32 sums, differs).
  * For tests and measurements; no counterpart in the reference.  Process-wide. */
-enum { MGEMV_MATRIX_CORE_AUTO = 0, MGEMV_MATRIX_CORE_REGISTER_OPERAND = 1, MGEMV_MATRIX_CORE_LDS_STAGED = 2 };
+enum {
+  MGEMV_MATRIX_CORE_AUTO = 0,
+  MGEMV_MATRIX_CORE_REGISTER_OPERAND = 1,
+  MGEMV_MATRIX_CORE_LDS_STAGED = 2,
+  MGEMV_MATRIX_CORE_K_STATIONARY = 3
+};
 MGEMV_API int mgemv_set_matrix_core_variant(int variant);
 
 /* The reference's kStages (mixed_gemv_test.cu:40; gemv/threadblock/default_dq_mma_simt.h:224-234 for
@@ -326,7 +335,8 @@ enum {
   MGEMV_KERNEL_AUTO = 0,
   MGEMV_KERNEL_VALU = 1,
   MGEMV_KERNEL_MATRIX_CORE_REGISTER_OPERAND = 2,
-  MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED = 3
+  MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED = 3,
+  MGEMV_KERNEL_MATRIX_CORE_K_STATIONARY = 4
 };
 typedef struct mgemv_tuned_plan {
   int n_out, k, weight_bits, group_size, m_batch; /* key */

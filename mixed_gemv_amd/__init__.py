@@ -39,6 +39,7 @@ from .api import (  # noqa: F401
     MATRIX_CORE_AUTO,
     MATRIX_CORE_REGISTER_OPERAND,
     MATRIX_CORE_LDS_STAGED,
+    MATRIX_CORE_K_STATIONARY,
     DEQUANT_AUTO,
     DEQUANT_EXACT_INTEGER,
     unpreprocess_weights,
@@ -52,6 +53,7 @@ from .api import (  # noqa: F401
     KERNEL_VALU,
     KERNEL_MATRIX_CORE_REGISTER_OPERAND,
     KERNEL_MATRIX_CORE_LDS_STAGED,
+    KERNEL_MATRIX_CORE_K_STATIONARY,
 )
 from . import autotune  # noqa: F401
 from ._lib import LIB_PATH, MixedGemvError  # noqa: F401

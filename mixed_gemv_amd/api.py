@@ -308,6 +308,7 @@ def set_matrix_core_threshold(min_m_batch=0):
 MATRIX_CORE_AUTO = 0
 MATRIX_CORE_REGISTER_OPERAND = 1
 MATRIX_CORE_LDS_STAGED = 2
+MATRIX_CORE_K_STATIONARY = 3
 
 
 def set_matrix_core_variant(variant=MATRIX_CORE_AUTO):
@@ -408,6 +409,7 @@ KERNEL_AUTO = 0
 KERNEL_VALU = 1
 KERNEL_MATRIX_CORE_REGISTER_OPERAND = 2
 KERNEL_MATRIX_CORE_LDS_STAGED = 3
+KERNEL_MATRIX_CORE_K_STATIONARY = 4
 
 
 def set_tuned_plan(n_out, k, weight_bits, group_size, m_batch, kernel=KERNEL_AUTO, split_k=0, tiles_per_wg=0,

@@ -20,7 +20,8 @@ from . import api
 _CACHE_BYTES = (256 << 20) + (32 << 20)
 _KERNEL_NAMES = {api.KERNEL_AUTO: "auto", api.KERNEL_VALU: "valu",
                  api.KERNEL_MATRIX_CORE_REGISTER_OPERAND: "matrix_core_register_operand",
-                 api.KERNEL_MATRIX_CORE_LDS_STAGED: "matrix_core_lds_staged"}
+                 api.KERNEL_MATRIX_CORE_LDS_STAGED: "matrix_core_lds_staged",
+                 api.KERNEL_MATRIX_CORE_K_STATIONARY: "matrix_core_k_stationary"}
 _installed = {}  # key tuple -> entry dict, what save_table writes
 
 
@@ -250,7 +251,8 @@ def _apply(cand):
                             cand.get("max_workgroups", 0))
     api.set_matrix_core_threshold({api.KERNEL_AUTO: 0, api.KERNEL_VALU: 17}.get(kernel, 1))
     api.set_matrix_core_variant({api.KERNEL_MATRIX_CORE_REGISTER_OPERAND: api.MATRIX_CORE_REGISTER_OPERAND,
-                                 api.KERNEL_MATRIX_CORE_LDS_STAGED: api.MATRIX_CORE_LDS_STAGED}
+                                 api.KERNEL_MATRIX_CORE_LDS_STAGED: api.MATRIX_CORE_LDS_STAGED,
+                                 api.KERNEL_MATRIX_CORE_K_STATIONARY: api.MATRIX_CORE_K_STATIONARY}
                                 .get(kernel, api.MATRIX_CORE_AUTO))
 
 

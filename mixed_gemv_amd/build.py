@@ -15,7 +15,7 @@ LINT_REPORT = os.path.join(LIB_DIR, "isa_lint.json")
 MIN_DOT_INSTRUCTIONS = 10000
 
 # One translation unit per family of kernel instantiations, so that they compile side by side.
-SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "gemv_kernels.hip", "probes.hip",
+SOURCES = ["launch_valu_f16.hip", "launch_valu_bf16.hip", "launch_mfma.hip", "launch_mfma_kstat.hip", "gemv_kernels.hip", "probes.hip",
            "host_utils.cpp"]
 
 # -ffp-contract=off: the dequantiser is a separately rounded fp16 multiply and add.
@@ -65,7 +65,8 @@ def lint_device_code(verbose=True):
 
 
 DEFAULT_PLANS = os.path.join(PKG_DIR, "default_plans.json")
-KERNEL_IDS = {"auto": 0, "valu": 1, "matrix_core_register_operand": 2, "matrix_core_lds_staged": 3}
+KERNEL_IDS = {"auto": 0, "valu": 1, "matrix_core_register_operand": 2, "matrix_core_lds_staged": 3,
+              "matrix_core_k_stationary": 4}
 
 
 def write_default_plans(path):

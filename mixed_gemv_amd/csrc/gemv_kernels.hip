@@ -172,6 +172,10 @@ PlanKnobs knobs_of_plan(const mgemv_tuned_plan& plan) {
       kn.matrix_core_min_batch = 1;
       kn.matrix_core_variant = MGEMV_MATRIX_CORE_LDS_STAGED;
       break;
+    case MGEMV_KERNEL_MATRIX_CORE_K_STATIONARY:
+      kn.matrix_core_min_batch = 1;
+      kn.matrix_core_variant = MGEMV_MATRIX_CORE_K_STATIONARY;
+      break;
     default: break;
   }
   return kn;
@@ -237,12 +241,68 @@ inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, boo
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Where the k-stationary matrix-core kernel (one wave per k step, one workgroup per compute unit walking
+// ceil(tiles / cus) tiles) is ahead of the others; int4 weights, fp16, at most 16 k steps.  Its waves hold their
+// activation operand in registers, so its loop has neither barriers nor LDS reads and costs the same at 1 to 8
+// rows; what it pays is a fixed start (operand through LDS, 0.8-1.6 us) and end (one barrier, one combine), so it
+// needs walks to spread them over, and tiles that divide evenly over the compute units.  Measured against the
+// built-in choice otherwise (us):
+//   2-8 rows, up to 8 k steps, walks from 2 tiles: 8192x4096 4 rows 6.06 / 6.88; 11008x4096 3 rows 7.29 / 8.80,
+//     8 rows 7.74 / 9.04; 14336x4096 4 rows 8.53 / 9.22; 22016x4096 2 rows 11.43 / 12.77; 28672x4096 8 rows
+//     13.92 / 15.50; 50304x2048 4 rows 13.98 / 15.61; 128256x4096 4 rows 46.3 / 50.2;
+//   2-8 rows, 9-16 k steps, walks from 3 tiles that fill their last round to within 12 %: 12288x8192 3 rows
+//     12.94 / 14.42; 16384x8192 4 rows 14.79 / 15.36; 28672x8192 2 / 4 / 8 rows 22.3 / 22.5 / 23.4 against 24.7 /
+//     24.9 / 26.2; 32768x8192 2 rows 25.6 / 27.6; but 8192x8192 (walks of 2) 11.7 / 11.2 at 4 rows and 14336x8192
+//     (3.5 tiles per compute unit) 16.0 / 15.3 at 8 rows the other way;
+//   1 row: only with 16 waves and walks from 7 tiles -- 28672x8192 22.2 / 22.5, 32768x8192 25.5 / 26.9, 57344x8192
+//     40.0 / 43.9 -- below that the VALU kernel's finer pipeline wins (16384x8192 14.9 / 13.1; 128256x4096, 8
+//     waves, 47.8 / 45.7);
+//   9-16 rows: the operand takes two rounds through LDS and twice the registers' worth of L2 traffic per wave;
+//     level with the LDS-staged kernel or behind it (28672x8192 25.4 / 26.4; 28672x4096 16.0 / 15.2), left to it.
+inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int cus) {
+  if (bits != 4 || m_batch > 8) return false;
+  const int walk = ceil_div(tiles, cus);
+  const long long padded = (long long)walk * cus * 100;
+  if (m_batch == 1) return ksteps > 8 && walk >= 7 && padded <= (long long)tiles * 105;
+  if (ksteps < 4 || (m_batch == 2 && ksteps < 8)) return false;
+  if (ksteps <= 8) return walk >= 2 && padded <= (long long)tiles * 115;
+  return walk >= 3 && padded <= (long long)tiles * 112;
+}
+
 LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs& knobs) {
   const int tiles = num_tiles(n_out), ksteps = num_ksteps(k, bits);
   const int cus = knobs.num_cus > 0 ? knobs.num_cus : kNumCus;  // the thresholds below were measured on 256 and scale with it
   const int ov_sk = knobs.split_k, ov_tw = knobs.tiles_per_wg;
   const int ov_t = knobs.tiles_per_wave;
   const bool mc = use_matrix_cores(m_batch, tiles, ksteps, knobs.matrix_core_min_batch, knobs.wide_waves, bits, cus);
+  // K-stationary kernel: one wave per k step (so at most 16 k steps), one workgroup per compute unit
+  // or fewer, each walking a contiguous run of tiles; more workgroups only where a walk's partial
+  // sums would not fit the LDS or its weights not a 32-bit offset.
+  const bool kstat_exists = ksteps <= kMaxWavesPerWorkgroup && !knobs.wide_waves;
+  const bool kstat_asked = mc && knobs.matrix_core_variant == MGEMV_MATRIX_CORE_K_STATIONARY;
+  const bool kstat_by_rule = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && knobs.matrix_core_min_batch == 0 &&
+                             ov_sk == 0 && ov_tw == 0 && ov_t == 0 && use_k_stationary(m_batch, tiles, ksteps, bits, cus);
+  if (kstat_exists && (kstat_asked || kstat_by_rule)) {
+    LaunchPlan lp{};
+    lp.matrix_core = true;
+    lp.k_stationary = true;
+    lp.split_k = ksteps;
+    lp.steps_per_wave = 1;
+    lp.tiles_per_wg = 1;
+    lp.tiles_per_wave = 1;
+    lp.stages = 2;
+    lp.workgroups = knobs.workgroups > 0 ? knobs.workgroups : cus;
+    if (lp.workgroups > tiles) lp.workgroups = tiles;
+    auto walk = [&]() { return ceil_div(tiles, lp.workgroups); };
+    const long long park_bytes = (long long)kKSlices * m_batch * kKStationaryParkSlots * 16;  // per tile of a walk
+    while (lp.workgroups < tiles &&
+           ((long long)walk() * ksteps * kUnitBytes >= (1ll << 31) || walk() * park_bytes > kMaxKStationaryLds))
+      lp.workgroups = lp.workgroups * 2 < tiles ? lp.workgroups * 2 : tiles;
+    lp.tiles_in_sequence = walk();
+    lp.wgs_per_xcd = ceil_div(lp.workgroups, kNumXcd);
+    lp.threads = kWave * lp.split_k;
+    return lp;
+  }
   // The LDS-staged kernel serves every matrix-core launch of two or more tiles.  (While its loop
   // still had a workgroup barrier per k step, the register-operand kernel was ahead on problems of
   // up to 256 tiles with up to 5 rows or up to 4 k steps; without the barrier the LDS-staged kernel
@@ -404,7 +464,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const int steps = ceil_div(ksteps, split_k);
   split_k = ceil_div(ksteps, steps);
   if (tiles_per_wg * split_k > max_waves) tiles_per_wg = max_waves / split_k;
-  LaunchPlan lp;
+  LaunchPlan lp{};
   lp.split_k = split_k;
   lp.tiles_per_wg = tiles_per_wg;
   lp.steps_per_wave = steps;
@@ -479,6 +539,13 @@ struct LaunchResources {
 LaunchResources launch_resources(const LaunchPlan& lp, int bits, int m_batch, int act) {
   LaunchResources r{};
   r.launches = 1;
+  if (lp.matrix_core && lp.k_stationary) {
+    r.max_threads = kWave * kMaxWavesPerWorkgroup;
+    const size_t stage = (size_t)lp.split_k * 8 * (step_k(bits) * 2 + 16), park = (size_t)lp.tiles_in_sequence * kKSlices * m_batch * kKStationaryParkSlots * 16;
+    // both when they fit (then no barrier stands between a wave's operand and its walk), else the larger of the two
+    r.lds_bytes = stage + park <= (size_t)kMaxKStationaryLds ? stage + park : stage > park ? stage : park;
+    return r;
+  }
   if (lp.matrix_core) {
     r.max_threads = kWave * kMaxWavesPerMfmaWorkgroup;
     if (lp.staged_rows != 0) {
@@ -613,6 +680,13 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
     g.tail.y = reinterpret_cast<half_t*>(y);
     g.tail.m_batch = m_batch;
     g.lds = launch_resources(g.plan, weight_bits, m_batch, act).lds_bytes;
+    if (g.plan.k_stationary) {
+      if (probe != kProbeNone) return MGEMV_ERR_QUANT_OP;  // no measurement builds of this kernel
+      const size_t stage = (size_t)g.plan.split_k * 8 * (step_k(weight_bits) * 2 + 16);
+      if (g.lds > stage && g.lds - stage >= (size_t)g.plan.tiles_in_sequence * kKSlices * m_batch * kKStationaryParkSlots * 16)
+        g.tail.flags |= kParkBehindStage;
+      return launch_mfma_kstat(g, weight_bits, quant_op, gpr, act) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+    }
     if (probe != kProbeNone) {
       const int rounds = g.plan.staged_rows != 0 ? g.plan.staged_rows / g.plan.tiles_per_wg : 0;
       if (probe == kProbeTimeline || rounds == 0 ||
@@ -942,7 +1016,7 @@ int mgemv_set_matrix_core_threshold(int min_m_batch) {
 
 int mgemv_set_matrix_core_variant(int variant) {
   if (variant != MGEMV_MATRIX_CORE_AUTO && variant != MGEMV_MATRIX_CORE_REGISTER_OPERAND &&
-      variant != MGEMV_MATRIX_CORE_LDS_STAGED)
+      variant != MGEMV_MATRIX_CORE_LDS_STAGED && variant != MGEMV_MATRIX_CORE_K_STATIONARY)
     return MGEMV_ERR_SIZE;
   mgemv::g_matrix_core_variant.store(variant);
   return MGEMV_OK;
@@ -979,7 +1053,7 @@ int mgemv_tuned_plan_set(const mgemv_tuned_plan* plan) {
   if (plan->element != MGEMV_ELEMENT_F16 && plan->element != MGEMV_ELEMENT_BF16) return MGEMV_ERR_QUANT_TYPE;
   const int t = plan->tiles_per_wave;
   if (t != 0 && t != 1 && t != 2 && t != 4) return MGEMV_ERR_SIZE;
-  if (plan->kernel < MGEMV_KERNEL_AUTO || plan->kernel > MGEMV_KERNEL_MATRIX_CORE_LDS_STAGED) return MGEMV_ERR_SIZE;
+  if (plan->kernel < MGEMV_KERNEL_AUTO || plan->kernel > MGEMV_KERNEL_MATRIX_CORE_K_STATIONARY) return MGEMV_ERR_SIZE;
   const mgemv::PlanKnobs kn = mgemv::knobs_of_plan(*plan);
   std::lock_guard<std::mutex> lock(mgemv::g_tuned_mutex);
   mgemv::g_tuned_plans[mgemv::PlanKey{plan->n_out, plan->k, plan->weight_bits, plan->group_size, plan->m_batch,
@@ -1049,7 +1123,7 @@ int mgemv_plan_coverage(int n_out, int m_batch, int k, int weight_bits, int grou
   const int grid = lp.wgs_per_xcd * kNumXcd;
   const int sequences = lp.workgroups * lp.tiles_per_wg;
   const int seq_base = tiles / sequences, seq_rem = tiles % sequences;  // as gemv_any passes them
-  const bool multi = !lp.matrix_core && lp.tiles_in_sequence > 1;
+  const bool multi = (!lp.matrix_core || lp.k_stationary) && lp.tiles_in_sequence > 1;
   const int rows = m_batch < kMaxValuBatch ? m_batch : kMaxValuBatch;
   std::vector<int> covered((size_t)tiles, 0);
   std::vector<char> block_seen((size_t)lp.workgroups, 0);
@@ -1060,7 +1134,7 @@ int mgemv_plan_coverage(int n_out, int m_batch, int k, int weight_bits, int grou
     if (block_seen[(size_t)wg]++) ++bad_ranges;   // two blocks with one logical id
     for (int ty = 0; ty < lp.tiles_per_wg; ++ty) {
       for (int kw = 0; kw < lp.split_k; ++kw) {
-        const WaveWork w = lp.matrix_core
+        const WaveWork w = lp.matrix_core && !lp.k_stationary
                                ? (lp.staged_rows != 0
                                       ? staged_wave_work(wg, ty, kw, lp.tiles_per_wg, tiles, lp.steps_per_wave, ksteps)
                                       : mfma_wave_work(lp.tiles_per_wave, wg, ty, kw, lp.tiles_per_wg, tiles,
@@ -1126,7 +1200,7 @@ int query_launch_any(int n_out, int m_batch, int k, int weight_bits, int group_s
   out[2] = lp.split_k;
   out[3] = lp.tiles_per_wg;
   out[4] = lp.steps_per_wave;
-  out[5] = !lp.matrix_core ? 0 : lp.staged_rows != 0 ? 2 : 1;
+  out[5] = !lp.matrix_core ? 0 : lp.k_stationary ? 3 : lp.staged_rows != 0 ? 2 : 1;
   out[6] = lp.tiles_per_wave;
   out[7] = lp.tiles_in_sequence;
   return MGEMV_OK;

@@ -18,9 +18,12 @@ constexpr int kMaxWavesPerWideWorkgroup = 8;  // VALU kernel with 3-4 activation
 constexpr int kMaxWavesPerMfmaWorkgroup = 8;  // leaves each wave of the matrix-core kernel 256 VGPRs
 constexpr int kNumXcd = 8;
 constexpr int kNumCus = 256;
+constexpr int kKStationaryParkSlots = kMaxWavesPerWorkgroup + 1;  // k-stationary matrix-core kernel: entries of 16 bytes per block of partial sums
+constexpr int kMaxKStationaryLds = 128 * 1024;  // most LDS the k-stationary matrix-core kernel parks partial sums in
 constexpr int kMaxValuBatch = 4;  // activation rows handled per launch by the VALU kernel
 constexpr int kExactIntegerFormOnly = 1;  // GemvTail::flags: never take the short int4 dequantiser
 constexpr int kSingleStage = 2;           // GemvTail::flags: no load in flight while a unit is computed (VALU kernel)
+constexpr int kParkBehindStage = 16;      // GemvTail::flags, k-stationary matrix-core kernel: the partial sums have LDS of their own behind the activation stages
 constexpr int kTimelineWaits = 8;         // GemvTail::flags, timeline probe: time the wait in front of every unit as well
 constexpr int kTimelineWordsPerWave = MGEMV_PROBE_TIMELINE_WORDS;  // 64-bit words the timeline probe writes per wave
 constexpr int kProbeNone = 0, kProbeLoadsOnly = 1, kProbeTimeline = 2, kProbeComputeOnly = 3;  // measurement builds of the VALU kernel
@@ -228,7 +231,8 @@ struct LaunchPlan {
   int tiles_in_sequence;  // VALU path: most tiles any wave walks one after the other
   int staged_rows;        // LDS-staged matrix-core kernel: 8 or 16 activation rows per stage; 0 = other kernels
   int stages;             // VALU path: 2 = the next unit is in flight while one is computed, 1 = it is not
-  bool matrix_core;       // one of the two matrix-core kernels (else the VALU kernel)
+  bool matrix_core;       // one of the matrix-core kernels (else the VALU kernel)
+  bool k_stationary;      // the matrix-core kernel whose waves keep one k step each while the workgroup walks tiles_in_sequence tiles
 };
 
 // Launches through hipLaunchKernel so that the status returned is this launch's own, not a
@@ -260,6 +264,7 @@ hipError_t launch_gemv_f16(const GemvLaunch& g, int bits, int qop, int mb, int g
 hipError_t launch_gemv_bf16(const GemvLaunch& g, int bits, int qop, int mb, int gpr);
 hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr);
 hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act);
+hipError_t launch_mfma_kstat(const GemvLaunch& g, int bits, int qop, int gpr, int act);
 // Measurement builds of the single-row int4 scale-and-zero fp16 VALU kernel (probe: kProbeLoadsOnly / kProbeTimeline / kProbeComputeOnly).
 hipError_t launch_gemv_probe(const GemvLaunch& g, int probe);
 // ... and of the LDS-staged matrix-core kernel (kProbeLoadsOnly / kProbeComputeOnly), where they exist.

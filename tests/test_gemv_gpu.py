@@ -212,7 +212,8 @@ def test_one_hot_activation_is_bit_exact_through_the_gemv_kernel(gpu):
 # (matrix-core variant, k-split waves, tiles per workgroup): the LDS-staged kernel with a stage per wave
 # (one tile per workgroup) and with stages shared by 2, 4 and 8 tiles, and the register-operand kernel
 MATRIX_CORE_LAUNCHES = [("lds_own_stages", "lds", 0, 1), ("lds_own_stages_split4", "lds", 4, 1), ("lds_shared_by_2", "lds", 2, 2),
-                        ("lds_shared_by_4", "lds", 2, 4), ("lds_shared_by_8", "lds", 1, 8), ("register_operand", "reg", 0, 0)]
+                        ("lds_shared_by_4", "lds", 2, 4), ("lds_shared_by_8", "lds", 1, 8), ("register_operand", "reg", 0, 0),
+                        ("k_stationary", "kstat", 0, 0)]
 
 
 @pytest.mark.parametrize("launch", MATRIX_CORE_LAUNCHES, ids=[c[0] for c in MATRIX_CORE_LAUNCHES])
@@ -220,9 +221,10 @@ MATRIX_CORE_LAUNCHES = [("lds_own_stages", "lds", 0, 1), ("lds_own_stages_split4
 def test_one_hot_rows_are_bit_exact_through_the_matrix_core_kernels(gpu, bits, launch):
     """Every activation row is a one-hot vector at a k of its own: y[b][n] == dq[n][k_b] bit for bit (up
     to the sign of a zero) through v_mfma_f32_16x16x32_f16 -- a product with 1 and sums with zeros are
-    exact in the matrix core too.  Pins the dequantiser inside both matrix-core kernels and which
+    exact in the matrix core too.  Pins the dequantiser inside the matrix-core kernels and which
     lane's weights meet which activation (the LDS stage's layout, 8 and 16 staged rows, shared and
-    own stages, the register operand's loads), which a tolerance against the VALU kernel does not."""
+    own stages, the register operand's loads, the k-stationary kernel's operand turned round through
+    LDS in one and two rounds), which a tolerance against the VALU kernel does not."""
     import torch
     _, variant, split, tw = launch
     k = 1536 if bits == 4 else 768
@@ -235,10 +237,11 @@ def test_one_hot_rows_are_bit_exact_through_the_matrix_core_kernels(gpu, bits, l
         dq = prob.oracle_dequant().view(np.uint16)
         try:
             mg.set_matrix_core_threshold(1)
-            mg.set_matrix_core_variant(mg.MATRIX_CORE_LDS_STAGED if variant == "lds" else mg.MATRIX_CORE_REGISTER_OPERAND)
-            mg.set_launch_override(split, tw, 0, 0)
+            mg.set_matrix_core_variant({"lds": mg.MATRIX_CORE_LDS_STAGED, "reg": mg.MATRIX_CORE_REGISTER_OPERAND,
+                                        "kstat": mg.MATRIX_CORE_K_STATIONARY}[variant])
+            mg.set_launch_override(split, tw, 0, 3 if variant == "kstat" else 0)   # k-stationary: walks of 2 and 3 tiles
             plan = mg.query_launch(prob.n_out, m_batch, k, bits)
-            assert plan["matrix_core"] == (2 if variant == "lds" else 1), plan
+            assert plan["matrix_core"] == {"lds": 2, "reg": 1, "kstat": 3}[variant], plan
             if variant == "lds" and tw:
                 assert plan["tiles_per_wg"] == tw, plan
             for trial in range(6):
@@ -434,7 +437,8 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
     assert np.array_equal(y_all.view(np.uint16), dev.run().view(np.uint16))
     assert mg.query_launch(80, m_batch, 2048, 4)["matrix_core"] == (0 if m_batch < 5 else 2)   # LDS-staged from 2 tiles
     assert mg.query_launch(16, 7, 2048, 4)["matrix_core"] == 1    # a single tile: register operand
-    assert mg.query_launch(8192, 7, 2048, 4)["matrix_core"] == 2
+    assert mg.query_launch(8192, 7, 2048, 4)["matrix_core"] == 3    # two tiles per compute unit: k-stationary
+    assert mg.query_launch(4096, 7, 2048, 4)["matrix_core"] == 2
     single = Problem("rows", 80, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True)
     for b in range(m_batch):
         single.x = prob.x[b:b + 1].copy()
@@ -593,7 +597,10 @@ RULES = [
     ("four_waves_from_16_k_steps", 9216, 8192, 1, dict(matrix_core=0, tiles_per_wg=1, split_k=4, steps_per_wave=4)),
     ("matrix_cores_at_3_rows", 5120, 4096, 3, dict(matrix_core=2)),
     ("two_tiles_even_split", 5120, 5120, 8, dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=5)),
-    ("two_tiles_592_workgroups", 18944, 3584, 8, dict(matrix_core=2, tiles_per_wg=2, workgroups=592)),
+    ("two_tiles_592_workgroups", 18944, 3584, 8, dict(matrix_core=2, tiles_per_wg=2, workgroups=592, variant="lds_staged")),
+    ("k_stationary_walks_of_5", 18944, 3584, 8, dict(matrix_core=3, workgroups=256, split_k=7, tiles_in_sequence=5)),
+    ("k_stationary_walks_of_3_16_waves", 12288, 8192, 3, dict(matrix_core=3, workgroups=256, split_k=16, tiles_in_sequence=3)),
+    ("k_stationary_two_rows", 22016, 4096, 2, dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=6)),
     ("four_tiles_160_workgroups", 10240, 8192, 8, dict(matrix_core=2, tiles_per_wg=4, workgroups=160)),
 ]
 
@@ -601,10 +608,16 @@ RULES = [
 @pytest.mark.parametrize("cfg", RULES, ids=[c[0] for c in RULES])
 def test_launch_rule_shapes_full_size(gpu, cfg):
     tag, n_out, k, mb, want = cfg
-    plan = mg.query_launch(n_out, mb, k, 4, 128)
-    assert {key: plan[key] for key in want} == want, plan
-    prob = Problem(tag, n_out, k, 4, SCALE_AND_ZEROS, 128, m_batch=mb, bias=(mb % 2 == 0), x_dist="normal")
-    check(prob, gpu, dequant=False)
+    want = dict(want)
+    # variant: the rule of the LDS-staged kernel on a shape that the k-stationary kernel now takes
+    mg.set_matrix_core_variant(mg.MATRIX_CORE_LDS_STAGED if want.pop("variant", None) else mg.MATRIX_CORE_AUTO)
+    try:
+        plan = mg.query_launch(n_out, mb, k, 4, 128)
+        assert {key: plan[key] for key in want} == want, plan
+        prob = Problem(tag, n_out, k, 4, SCALE_AND_ZEROS, 128, m_batch=mb, bias=(mb % 2 == 0), x_dist="normal")
+        check(prob, gpu, dequant=False)
+    finally:
+        mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
 
 
 @pytest.mark.parametrize("cfg", FULL, ids=[c[0] for c in FULL])
@@ -617,15 +630,16 @@ def test_baseline_configs_full_size(gpu, cfg):
 
 def test_hip_graph_replays_match_eager_launches(gpu):
     """The entry points neither allocate nor synchronise, so a caller may capture them; every replay of
-    a graph holding a VALU launch, both matrix-core launches and a bf16 launch must reproduce the eager
+    a graph holding a VALU launch, the three matrix-core launches and a bf16 launch must reproduce the eager
     results bit for bit, with eager work and synchronisations between the replays."""
     import torch
     probs = [Problem("g_valu", 320, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=2, bias=True),
              Problem("g_reg", 16, 2048, 4, SCALE_AND_ZEROS, 64, m_batch=6, bias=True),       # one tile: register-operand matrix core
              Problem("g_lds", 320, 2048, 8, PER_COLUMN, 0, m_batch=16, bias=False),          # LDS-staged, 16 rows staged
+             Problem("g_kstat", 8192, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=3, bias=True),   # walks of 2 tiles: k-stationary
              Problem("g_bf16", 320, 2048, 4, SCALE_AND_ZEROS, 128, m_batch=1, bias=True, element="bf16")]
     devs = [DeviceProblem(p, gpu) for p in probs]
-    assert [mg.query_launch(p.n_out, p.m_batch, 2048, p.bits)["matrix_core"] for p in probs[:3]] == [0, 1, 2]
+    assert [mg.query_launch(p.n_out, p.m_batch, 2048, p.bits)["matrix_core"] for p in probs[:4]] == [0, 1, 2, 3]
     eager = [d.run().copy() for d in devs]
 
     def launch_all():

@@ -212,7 +212,7 @@ def test_gemv_argument_checks_return_codes_without_launching():
     assert lib.mgemv_set_launch_override(-1, 0, 0, 0) == 10
     assert lib.mgemv_set_launch_override(0, 0, 3, 0) == 10
     assert lib.mgemv_set_matrix_core_threshold(18) == 8
-    assert lib.mgemv_set_matrix_core_variant(3) == 10 and lib.mgemv_set_matrix_core_variant(0) == 0
+    assert lib.mgemv_set_matrix_core_variant(4) == 10 and lib.mgemv_set_matrix_core_variant(0) == 0
     assert lib.mgemv_set_dequant_form(2) == 10 and lib.mgemv_set_dequant_form(0) == 0
 
 
@@ -354,7 +354,7 @@ def test_tuned_plan_table_steers_exactly_its_problem(tmp_path):
         assert mg.query_launch(11008, 1, 4096, 4, 128) == want
         # argument checks
         for bad, code in ((dict(weight_bits=5), 7), (dict(n_out=0), 10), (dict(group_size=-1), 5), (dict(m_batch=0), 8),
-                          (dict(m_batch=17), 8), (dict(kernel=4), 10), (dict(tiles_per_wave=3), 10), (dict(split_k=-1), 10)):
+                          (dict(m_batch=17), 8), (dict(kernel=5), 10), (dict(tiles_per_wave=3), 10), (dict(split_k=-1), 10)):
             args = dict(n_out=64, k=512, weight_bits=4, group_size=128, m_batch=1)
             args.update(bad)
             with pytest.raises(MixedGemvError) as ei:
@@ -411,7 +411,10 @@ def test_adaptor_mirror_rejects_small_groups_like_the_reference():
 # test pins the rules, so a change to plan_launch that moves one of them shows up here.
 BUILTIN_PLANS = [
     # exact fit: one 4-wave workgroup per compute unit, every wave walking 7 tiles
-    ((28672, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256, split_k=4, tiles_in_sequence=7)),
+    ((28672, 1, 4096), dict(matrix_core=0, workgroups=256, threads=256, split_k=4, tiles_in_sequence=7)),
+    # ... and with 9-16 k steps and walks of 7 tiles or more, the k-stationary matrix-core kernel: one wave per k step
+    ((28672, 1, 8192), dict(matrix_core=3, workgroups=256, threads=1024, split_k=16, steps_per_wave=1, tiles_in_sequence=7)),
+    ((16384, 1, 8192), dict(matrix_core=0, workgroups=256, tiles_per_wg=4)),                   # walks of 4: the VALU kernel
     ((8192, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256)),
     # at most one workgroup per compute unit: four k-split waves
     ((4096, 1, 4096), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=2)),
@@ -446,30 +449,48 @@ BUILTIN_PLANS = [
     ((4096, 4, 14336), dict(matrix_core=2, tiles_per_wg=1)),   # 4 rows, 129-256 tiles, from 16 k steps
     ((2048, 4, 8192), dict(matrix_core=0)),
     ((10240, 2, 8192), dict(matrix_core=0)),
-    ((28672, 2, 8192), dict(matrix_core=2)),
+    ((28672, 2, 8192), dict(matrix_core=2, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((50304, 2, 2048), dict(matrix_core=0)),
     ((151936, 2, 2048), dict(matrix_core=2)),
+    # 2-8 rows on the k-stationary kernel: walks of 2 tiles or more with up to 8 k steps (2 rows: 8 k steps), of 3 or
+    # more with 9-16, that fill their last round; one workgroup per compute unit, one wave per k step
+    ((28672, 2, 8192), dict(matrix_core=3, workgroups=256, split_k=16, tiles_in_sequence=7)),
+    ((11008, 3, 4096), dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=3)),
+    ((8192, 8, 4096), dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=2)),
+    ((8192, 7, 2048), dict(matrix_core=3, workgroups=256, split_k=4, tiles_in_sequence=2)),
+    ((22016, 2, 4096), dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=6)),
+    ((12288, 3, 8192), dict(matrix_core=3, workgroups=256, split_k=16, tiles_in_sequence=3)),
+    ((8192, 8, 8192), dict(matrix_core=2)),                    # walks of 2 with 16 k steps: no
+    ((14336, 8, 8192), dict(matrix_core=2)),                   # 3.5 tiles per compute unit: no
+    ((32768, 4, 1024), dict(matrix_core=2)),                   # 2 k steps, 2 waves per compute unit: no
+    ((28672, 9, 8192), dict(matrix_core=2)),                   # 9 rows and more: no
+    ((128256, 8, 4096), dict(matrix_core=3, workgroups=1024, tiles_in_sequence=8)),   # the partial sums of a walk must fit the LDS
     # tiles that share an activation stage: as few as give at most 256 workgroups ...
     ((5120, 8, 5120), dict(matrix_core=2, tiles_per_wg=2, workgroups=160, split_k=2, steps_per_wave=5)),
     ((8192, 16, 8192), dict(matrix_core=2, tiles_per_wg=2, workgroups=256, split_k=4)),
     ((10240, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=160)),
     ((28672, 16, 8192), dict(matrix_core=2, tiles_per_wg=8, workgroups=224, split_k=1)),
     # ... or, when that cannot be had, a count whose last round of 256 is well filled
-    ((28672, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=448)),
-    ((18944, 8, 3584), dict(matrix_core=2, tiles_per_wg=2, workgroups=592, split_k=1)),
+    ((28672, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=448, variant=mg.MATRIX_CORE_LDS_STAGED)),
+    ((18944, 8, 3584), dict(matrix_core=2, tiles_per_wg=2, workgroups=592, split_k=1, variant=mg.MATRIX_CORE_LDS_STAGED)),
     # an uneven k split is halved only while the workgroup keeps four waves
     ((4096, 8, 6656), dict(matrix_core=2, tiles_per_wg=1, split_k=4, steps_per_wave=4)),
     ((8192, 8, 6656), dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=7)),
 ]
 
 
-@pytest.mark.parametrize("shape,want", BUILTIN_PLANS, ids=[f"{s[0]}x{s[2]}_m{s[1]}" for s, _ in BUILTIN_PLANS])
+@pytest.mark.parametrize("shape,want", BUILTIN_PLANS,
+                         ids=[f"{s[0]}x{s[2]}_m{s[1]}" + ("_lds_staged" if "variant" in w else "") for s, w in BUILTIN_PLANS])
 def test_builtin_launch_rules_on_the_shapes_they_were_measured_on(shape, want):
+    """variant: the rules of the named matrix-core kernel, on a shape that the k-stationary kernel now takes."""
     n_out, m_batch, k = shape
+    want = dict(want)
     mg.set_default_plans(False)   # the rules themselves, without the built-in table of measured exceptions
+    mg.set_matrix_core_variant(want.pop("variant", mg.MATRIX_CORE_AUTO))
     try:
         got = mg.query_launch(n_out, m_batch, k, 4, 128)
     finally:
+        mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
         mg.set_default_plans(True)
     assert {key: got[key] for key in want} == want, got
     # every plan covers every tile and every k step, within the workgroup size the kernels allow
@@ -510,8 +531,8 @@ def test_default_plan_table_is_the_shipped_json_and_applies_to_256_compute_units
     path = os.path.join(os.path.dirname(_lib.LIB_PATH), "..", "default_plans.json")
     with open(path) as f:
         table = json.load(f)
-    assert table["format"] == 1 and mg.default_plan_count() == len(table["plans"]) >= 1
-    kinds = {0: 0, 1: 0, 2: 1, 3: 2}   # MGEMV_KERNEL_* -> what query_launch reports as matrix_core
+    assert table["format"] == 1 and mg.default_plan_count() == len(table["plans"])   # (it may be empty)
+    kinds = {0: 0, 1: 0, 2: 1, 3: 2, 4: 3}   # MGEMV_KERNEL_* -> what query_launch reports as matrix_core
     for e in table["plans"]:
         key = (e["n_out"], e["m_batch"], e["k"], e["weight_bits"], e["group_size"])
         got = mg.query_launch(*key, element=e["element"], num_compute_units=256)

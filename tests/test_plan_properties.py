@@ -77,8 +77,8 @@ def test_built_in_plans_cover_every_problem():
         cus = int(rng.choice(DEVICE_SIZES))
         q, _ = check_plan(*prob, cus)
         kinds.add((q["matrix_core"], q["tiles_in_sequence"] > 1, q["tiles_per_wg"] > 1))
-    # the sample reaches every kind of launch: VALU with and without walks and tile pairs, both matrix-core kernels
-    assert {k[0] for k in kinds} == {0, 2} or {k[0] for k in kinds} == {0, 1, 2}
+    # the sample reaches every kind of launch: VALU with and without walks and tile pairs, the matrix-core kernels
+    assert {k[0] for k in kinds} == {0, 2, 3} or {k[0] for k in kinds} == {0, 1, 2, 3}
     assert (0, True, False) in kinds and (0, False, True) in kinds and (0, True, True) in kinds
 
 
@@ -89,7 +89,7 @@ def test_every_override_combination_still_covers():
         for tiles_per_wg in (0, 1, 2, 4, 8):
             for tiles_per_wave in (0, 1, 2, 4):
                 for max_wg in (0, 1, 100, 256, 512):
-                    for threshold, variant in ((0, 0), (17, 0), (1, 1), (1, 2), (2, 0)):
+                    for threshold, variant in ((0, 0), (17, 0), (1, 1), (1, 2), (2, 0), (1, 3)):
                         stages = int(rng.integers(0, 3))
                         with overrides(split_k, tiles_per_wg, tiles_per_wave, max_wg, threshold, variant, stages):
                             for _ in range(4):
