@@ -843,7 +843,7 @@ def main():
             # config 5 names 8 distinct rotated buffers: all of them are checked, not only the first
             sets = list(range(w2.sets)) if (base == "c5" and rows is None) else [0]
             entry["parity"] = parity_summary(w2, sets, threads, with_dequant=(rows in (None, 1)))
-        if base == "c5" and element == "f16" and batch == 1 and not args.no_ceilings:
+        if base == "c5" and rows is None and element == "f16" and batch == 1 and not args.no_ceilings:
             out.setdefault("ceilings", {})[base] = ceilings_of(w2, use_graph, timeline=True)
         if base == "c4" and rows in (8, 16) and element == "f16" and batch == 1 and not args.no_ceilings:
             c = ceilings_of_rows(w2, use_graph)

@@ -241,32 +241,69 @@ inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, boo
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Tiles per workgroup of the LDS-staged matrix-core kernel (= waves that share one activation stage): as few as
+// bring the launch down to one workgroup per compute unit or fewer, at most 8 and at most a quarter of the staged
+// rows.  Measured, 16 rows: 4096x4096 (256 tiles) 6.3 us at 1 tile against 7.2 at 2; 8192x8192 (512)
+// 13.4 at 2 against 17.8 at 4; 11008x4096 (688) 10.1 at 4 against 11.3 at 2 and 14.2 at 8;
+// 28672x8192 (1792) 28.3 at 8 against 30.6 at 4 and 32.8 at 2.  8 rows: 4096x4096 5.4 at 1
+// against 6.4 at 2; 5120x5120 (320) 7.7 at 2 against 9.3 at 1; 10240x8192 (640) 14.7 at 4
+// against 15.5 at 2; 11008x4096 9.0 at 4 against 9.7 at 2; 28672x8192 27.6 at 4 against 29.5 at 2.
+// Still more workgroups than compute units: a count just above a multiple of 256 leaves most
+// of the last round idle, and halving the tiles per workgroup evens that out (18944x3584,
+// 8 rows: 296 workgroups of 4 tiles 12.8 us, 592 of 2 tiles 11.8; 22016x4096: 14.4 / 13.3):
+// the largest count whose last round is at least three quarters full.
+inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
+  int tw = 1;
+  while (ceil_div(tiles, tw) > cus && tw * 2 <= 8 && tw * 4 <= staged_rows) tw *= 2;
+  if (ceil_div(tiles, tw) > cus) {
+    for (int t = tw; t >= 1; t /= 2) {
+      const int wgs = ceil_div(tiles, t);
+      if (wgs * 4 >= ceil_div(wgs, cus) * cus * 3) return t;
+    }
+  }
+  return tw;
+}
+
 // Where the k-stationary matrix-core kernel (one wave per k step, one workgroup per compute unit walking
-// ceil(tiles / cus) tiles) is ahead of the others; int4 weights, fp16, at most 16 k steps.  Its waves hold their
-// activation operand in registers, so its loop has neither barriers nor LDS reads and costs the same at 1 to 8
-// rows; what it pays is a fixed start (operand through LDS, 0.8-1.6 us) and end (one barrier, one combine), so it
-// needs walks to spread them over, and tiles that divide evenly over the compute units.  Measured against the
-// built-in choice otherwise (us):
-//   2-8 rows, up to 8 k steps, walks from 2 tiles: 8192x4096 4 rows 6.06 / 6.88; 11008x4096 3 rows 7.29 / 8.80,
-//     8 rows 7.74 / 9.04; 14336x4096 4 rows 8.53 / 9.22; 22016x4096 2 rows 11.43 / 12.77; 28672x4096 8 rows
-//     13.92 / 15.50; 50304x2048 4 rows 13.98 / 15.61; 128256x4096 4 rows 46.3 / 50.2;
-//   2-8 rows, 9-16 k steps, walks from 3 tiles that fill their last round to within 12 %: 12288x8192 3 rows
-//     12.94 / 14.42; 16384x8192 4 rows 14.79 / 15.36; 28672x8192 2 / 4 / 8 rows 22.3 / 22.5 / 23.4 against 24.7 /
-//     24.9 / 26.2; 32768x8192 2 rows 25.6 / 27.6; but 8192x8192 (walks of 2) 11.7 / 11.2 at 4 rows and 14336x8192
-//     (3.5 tiles per compute unit) 16.0 / 15.3 at 8 rows the other way;
-//   1 row: only with 16 waves and walks from 7 tiles -- 28672x8192 22.2 / 22.5, 32768x8192 25.5 / 26.9, 57344x8192
-//     40.0 / 43.9 -- below that the VALU kernel's finer pipeline wins (16384x8192 14.9 / 13.1; 128256x4096, 8
-//     waves, 47.8 / 45.7);
+// ceil(tiles / cus) tiles) is ahead of the others; int4 weights, fp16, 4 to 16 k steps, up to 8 rows.  Its waves hold
+// their activation operand in registers, so its loop has neither barriers nor LDS reads and costs the same at 1 to
+// 8 rows; what it pays is a fixed start (operand through LDS, 0.8-1.6 us) and end (one barrier, one combine), and a
+// tail: when the weight stream ends, every wave of a SIMD still has a unit to compute.  Measured against the
+// built-in choice otherwise (us, k-stationary first):
+//   up to 8 k steps (at most 2 waves per SIMD), 3-8 rows, more tiles than compute units (4-5 k steps: 1.5 times
+//     as many; 2 rows: 8 k steps and 2.5 times as many): 4608x4096 4 rows 5.60 / 6.41; 5120x3072 5.52 / 6.82; 8192x4096 6.06 / 6.88;
+//     10240x4096 7.25 / 8.77, 8 rows 7.66 / 8.89; 11008x4096 3 rows 7.29 / 8.80; 22016x4096 2 rows 11.43 / 12.77;
+//     28672x4096 8 rows 13.92 / 15.50; 8192x2048 7 rows 4.75 / 5.17; 50304x2048 4 rows 13.98 / 15.61; 128256x4096
+//     4 rows 46.3 / 50.2; but 4608x2048 4 rows 4.58 / 4.49, and with 1-2 k steps there are 1-2 waves per compute
+//     unit (32768x1024 10.4 / 7.2);
+//   9-16 k steps: wherever its one-workgroup-per-compute-unit walks fill the machine better than the LDS-staged
+//     kernel's workgroups of 1-4 tiles do -- 9216x8192 4 rows 12.48 / 14.18; 10240x8192 12.65 / 14.14, 8 rows 13.37
+//     / 14.49; 12288x8192 3 rows 12.94 / 14.42; 18432x8192 17.73 / 22.40; 20480x8192 18.23 / 22.61; 28672x8192 2 /
+//     4 / 8 rows 22.3 / 22.5 / 23.4 against 24.7 / 24.9 / 26.2 -- and, where the two fill it alike: at 3-4 rows with
+//     walks of up to 3 tiles or tiles that divide evenly (5120x5120 6.82 / 7.62; 8192x7168 8.79 / 10.03; 8192x8192
+//     10.34 / 10.37; 16384x8192 14.79 / 15.36; but 13312x8192 14.99 / 14.63, 13824x5120 10.97 / 10.60), at 5-8 rows
+//     only up to 12 k steps with walks of 2 (8192x6144 7.80 / 8.64; but 8192x8192 11.01 / 10.50, 16384x8192 16.42 /
+//     15.95, 14336x8192 16.0 / 15.3), at 2 rows from walks of 3 (12288x8192 12.74 / 13.28; 8192x8192 9.93 / 9.05);
+//   1 row: only with 9-16 k steps and walks from 7 tiles -- 28672x8192 22.2 / 22.5 (three leases: 1.9, 1.8, 0.5 %
+//     ahead), 32768x8192 25.5 / 26.9, 57344x8192 40.0 / 43.9 -- below that the VALU kernel's finer pipeline wins
+//     (16384x8192 14.9 / 13.1; 128256x4096, 8 waves, 47.8 / 45.7);
 //   9-16 rows: the operand takes two rounds through LDS and twice the registers' worth of L2 traffic per wave;
 //     level with the LDS-staged kernel or behind it (28672x8192 25.4 / 26.4; 28672x4096 16.0 / 15.2), left to it.
 inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int cus) {
-  if (bits != 4 || m_batch > 8) return false;
+  if (bits != 4 || m_batch > 8 || ksteps < 4) return false;
   const int walk = ceil_div(tiles, cus);
-  const long long padded = (long long)walk * cus * 100;
-  if (m_batch == 1) return ksteps > 8 && walk >= 7 && padded <= (long long)tiles * 105;
-  if (ksteps < 4 || (m_batch == 2 && ksteps < 8)) return false;
-  if (ksteps <= 8) return walk >= 2 && padded <= (long long)tiles * 115;
-  return walk >= 3 && padded <= (long long)tiles * 112;
+  const long long slots = (long long)walk * cus;  // tiles the launch has room for
+  if (m_batch == 1) return ksteps > 8 && walk >= 7 && slots * 100 <= (long long)tiles * 105;
+  if (ksteps <= 8) {
+    if (m_batch == 2) return ksteps == 8 && tiles * 2 >= cus * 5;  // the VALU kernel's two rows are cheap: 8192x4096 5.90 / 5.95
+    return ksteps <= 5 ? tiles * 2 >= cus * 3 : tiles > cus;
+  }
+  const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);
+  const long long lds_slots = (long long)ceil_div(ceil_div(tiles, tw), cus) * cus * tw;
+  if (lds_slots * 10 >= slots * 11) return m_batch >= 3 || walk >= 3;  // fills the machine better by a tenth or more
+  if (m_batch == 2) return walk == 3 || (walk > 3 && slots == tiles);
+  if (m_batch <= 4) return walk == 2 || walk == 3 || slots == tiles;
+  return walk == 2 && ksteps <= 12;
 }
 
 LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs& knobs) {
@@ -278,6 +315,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   // K-stationary kernel: one wave per k step (so at most 16 k steps), one workgroup per compute unit
   // or fewer, each walking a contiguous run of tiles; more workgroups only where a walk's partial
   // sums would not fit the LDS or its weights not a 32-bit offset.
+  // fp16 only: the bf16 dequantiser does not fit 128 registers beside the operand (with spills: 28672x8192 40.2 us against 35.1)
   const bool kstat_exists = ksteps <= kMaxWavesPerWorkgroup && !knobs.wide_waves;
   const bool kstat_asked = mc && knobs.matrix_core_variant == MGEMV_MATRIX_CORE_K_STATIONARY;
   const bool kstat_by_rule = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && knobs.matrix_core_min_batch == 0 &&
@@ -316,30 +354,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     LaunchPlan lp{};
     lp.matrix_core = true;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
-    // Tiles per workgroup = waves that share one activation stage: as few as bring the launch down
-    // to one workgroup per compute unit or fewer, at most 8 and at most half the staged rows.
-    // Measured, 16 rows: 4096x4096 (256 tiles) 6.3 us at 1 tile against 7.2 at 2; 8192x8192 (512)
-    // 13.4 at 2 against 17.8 at 4; 11008x4096 (688) 10.1 at 4 against 11.3 at 2 and 14.2 at 8;
-    // 28672x8192 (1792) 28.3 at 8 against 30.6 at 4 and 32.8 at 2.  8 rows: 4096x4096 5.4 at 1
-    // against 6.4 at 2; 5120x5120 (320) 7.7 at 2 against 9.3 at 1; 10240x8192 (640) 14.7 at 4
-    // against 15.5 at 2; 11008x4096 9.0 at 4 against 9.7 at 2; 28672x8192 27.6 at 4 against 29.5 at 2.
-    lp.tiles_per_wg = 1;
-    while (ceil_div(tiles, lp.tiles_per_wg) > cus && lp.tiles_per_wg * 2 <= 8 &&
-           lp.tiles_per_wg * 4 <= lp.staged_rows)
-      lp.tiles_per_wg *= 2;
-    // Still more workgroups than compute units: a count just above a multiple of 256 leaves most
-    // of the last round idle, and halving the tiles per workgroup evens that out (18944x3584,
-    // 8 rows: 296 workgroups of 4 tiles 12.8 us, 592 of 2 tiles 11.8; 22016x4096: 14.4 / 13.3).
-    // Largest count whose last round is at least three quarters full.
-    if (ceil_div(tiles, lp.tiles_per_wg) > cus) {
-      for (int tw = lp.tiles_per_wg; tw >= 1; tw /= 2) {
-        const int wgs = ceil_div(tiles, tw);
-        if (wgs * 4 >= ceil_div(wgs, cus) * cus * 3) {
-          lp.tiles_per_wg = tw;
-          break;
-        }
-      }
-    }
+    lp.tiles_per_wg = lds_staged_tiles_per_wg(tiles, lp.staged_rows, cus);
     // the kernel exists for 2, 4, 8 or 16 staged rows per wave of a k range
     if (ov_tw > 0 && ov_tw <= 8 && lp.staged_rows % ov_tw == 0 && lp.staged_rows / ov_tw >= 2) lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);

@@ -595,13 +595,15 @@ RULES = [
     ("paired_tiles", 5120, 5120, 1, dict(matrix_core=0, tiles_per_wg=2, split_k=2, workgroups=160)),
     ("paired_tiles_m2_long_k", 7168, 14336, 2, dict(matrix_core=0, tiles_per_wg=2, split_k=2, steps_per_wave=14)),
     ("four_waves_from_16_k_steps", 9216, 8192, 1, dict(matrix_core=0, tiles_per_wg=1, split_k=4, steps_per_wave=4)),
-    ("matrix_cores_at_3_rows", 5120, 4096, 3, dict(matrix_core=2)),
-    ("two_tiles_even_split", 5120, 5120, 8, dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=5)),
+    ("matrix_cores_at_3_rows", 5120, 4096, 3, dict(matrix_core=2, variant="lds_staged")),
+    ("two_tiles_even_split", 5120, 5120, 8, dict(matrix_core=2, tiles_per_wg=2, split_k=2, steps_per_wave=5, variant="lds_staged")),
     ("two_tiles_592_workgroups", 18944, 3584, 8, dict(matrix_core=2, tiles_per_wg=2, workgroups=592, variant="lds_staged")),
     ("k_stationary_walks_of_5", 18944, 3584, 8, dict(matrix_core=3, workgroups=256, split_k=7, tiles_in_sequence=5)),
     ("k_stationary_walks_of_3_16_waves", 12288, 8192, 3, dict(matrix_core=3, workgroups=256, split_k=16, tiles_in_sequence=3)),
     ("k_stationary_two_rows", 22016, 4096, 2, dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=6)),
-    ("four_tiles_160_workgroups", 10240, 8192, 8, dict(matrix_core=2, tiles_per_wg=4, workgroups=160)),
+    ("four_tiles_160_workgroups", 10240, 8192, 8, dict(matrix_core=2, tiles_per_wg=4, workgroups=160, variant="lds_staged")),
+    ("k_stationary_better_filled", 10240, 8192, 8, dict(matrix_core=3, workgroups=256, tiles_in_sequence=3)),
+    ("k_stationary_walks_of_2", 5120, 4096, 3, dict(matrix_core=3, workgroups=256, tiles_in_sequence=2)),
 ]
 
 

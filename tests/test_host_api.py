@@ -444,11 +444,12 @@ BUILTIN_PLANS = [
     ((4096, 5, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
     ((16, 8, 4096), dict(matrix_core=1)),                      # a single tile: the register-operand kernel
     ((4096, 8, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
-    ((5120, 3, 4096), dict(matrix_core=2)),
+    ((5120, 3, 4096), dict(matrix_core=2, variant=mg.MATRIX_CORE_LDS_STAGED)),
+    ((5120, 3, 4096), dict(matrix_core=3, workgroups=256, tiles_in_sequence=2)),
     ((4096, 3, 14336), dict(matrix_core=0)),
     ((4096, 4, 14336), dict(matrix_core=2, tiles_per_wg=1)),   # 4 rows, 129-256 tiles, from 16 k steps
     ((2048, 4, 8192), dict(matrix_core=0)),
-    ((10240, 2, 8192), dict(matrix_core=0)),
+    ((10240, 2, 8192), dict(matrix_core=0, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((28672, 2, 8192), dict(matrix_core=2, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((50304, 2, 2048), dict(matrix_core=0)),
     ((151936, 2, 2048), dict(matrix_core=2)),
@@ -460,15 +461,25 @@ BUILTIN_PLANS = [
     ((8192, 7, 2048), dict(matrix_core=3, workgroups=256, split_k=4, tiles_in_sequence=2)),
     ((22016, 2, 4096), dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=6)),
     ((12288, 3, 8192), dict(matrix_core=3, workgroups=256, split_k=16, tiles_in_sequence=3)),
-    ((8192, 8, 8192), dict(matrix_core=2)),                    # walks of 2 with 16 k steps: no
-    ((14336, 8, 8192), dict(matrix_core=2)),                   # 3.5 tiles per compute unit: no
+    ((10240, 8, 8192), dict(matrix_core=3, tiles_in_sequence=3)),    # 640 tiles: better filled than 160 workgroups of 4 tiles
+    ((10240, 2, 8192), dict(matrix_core=3, tiles_in_sequence=3)),
+    ((5120, 8, 5120), dict(matrix_core=3, tiles_in_sequence=2)),     # 10 k steps, walks of 2
+    ((8192, 4, 8192), dict(matrix_core=3, tiles_in_sequence=2)),     # 3-4 rows: walks of 2 and 3, or tiles that divide evenly
+    ((16384, 4, 8192), dict(matrix_core=3, tiles_in_sequence=4)),
+    ((13312, 4, 8192), dict(matrix_core=2)),                   # walks of 4 that neither divide evenly nor fill better: no
+    ((8192, 8, 8192), dict(matrix_core=2)),                    # 5-8 rows, 16 k steps, filled alike: no
+    ((16384, 8, 8192), dict(matrix_core=2)),
+    ((14336, 8, 8192), dict(matrix_core=2)),
+    ((8192, 2, 8192), dict(matrix_core=0)),                    # 2 rows on walks of 2: the VALU kernel
+    ((6144, 2, 4096), dict(matrix_core=0)),
+    ((4608, 4, 2048), dict(matrix_core=0)),                    # 4 k steps: from 1.5 tiles per compute unit
     ((32768, 4, 1024), dict(matrix_core=2)),                   # 2 k steps, 2 waves per compute unit: no
     ((28672, 9, 8192), dict(matrix_core=2)),                   # 9 rows and more: no
     ((128256, 8, 4096), dict(matrix_core=3, workgroups=1024, tiles_in_sequence=8)),   # the partial sums of a walk must fit the LDS
     # tiles that share an activation stage: as few as give at most 256 workgroups ...
-    ((5120, 8, 5120), dict(matrix_core=2, tiles_per_wg=2, workgroups=160, split_k=2, steps_per_wave=5)),
+    ((5120, 8, 5120), dict(matrix_core=2, tiles_per_wg=2, workgroups=160, split_k=2, steps_per_wave=5, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((8192, 16, 8192), dict(matrix_core=2, tiles_per_wg=2, workgroups=256, split_k=4)),
-    ((10240, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=160)),
+    ((10240, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=160, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((28672, 16, 8192), dict(matrix_core=2, tiles_per_wg=8, workgroups=224, split_k=1)),
     # ... or, when that cannot be had, a count whose last round of 256 is well filled
     ((28672, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=448, variant=mg.MATRIX_CORE_LDS_STAGED)),

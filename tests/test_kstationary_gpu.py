@@ -149,12 +149,15 @@ def test_the_built_in_rule_takes_it_where_it_was_measured_ahead(gpu):
     import torch
     cus = torch.cuda.get_device_properties(gpu).multi_processor_count
     n_out = 16 * 2 * cus
-    for rows, k in ((4, 4096), (8, 2048), (2, 4096)):
+    for rows, k, walk in ((4, 4096, 2), (8, 2048, 2), (2, 4096, 3)):     # 2 rows: from 2.5 tiles per compute unit
+        n_out = 16 * walk * cus
         plan = mg.query_launch(n_out, rows, k, 4, 128, num_compute_units=cus)
-        assert plan["matrix_core"] == 3 and plan["workgroups"] == -(-cus // 8) * 8 and plan["tiles_in_sequence"] == 2, plan
+        assert plan["matrix_core"] == 3 and plan["workgroups"] == -(-cus // 8) * 8 and plan["tiles_in_sequence"] == walk, plan
         prob = Problem("ks_rule", n_out, k, 4, SCALE_AND_ZEROS, 128, m_batch=rows, bias=True, x_dist="normal")
         _, rel, _ = error_report(DeviceProblem(prob, gpu).run(), prob.oracle_gemv(threads=16))
         assert rel <= REL_TOL, (rows, k, rel)
+    n_out = 16 * 2 * cus
+    assert mg.query_launch(n_out, 2, 4096, 4, 128, num_compute_units=cus)["matrix_core"] == 0     # 2 rows on walks of 2: VALU
     assert mg.query_launch(n_out, 16, 4096, 4, 128, num_compute_units=cus)["matrix_core"] == 2    # 9-16 rows: LDS-staged
     assert mg.query_launch(n_out, 4, 1024, 4, 128, num_compute_units=cus)["matrix_core"] != 3      # 2 k steps: too few waves
     assert mg.query_launch(n_out, 4, 16384, 4, 128, num_compute_units=cus)["matrix_core"] == 2     # 32 k steps: no such launch
