@@ -247,15 +247,22 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
                                         int max_workgroups);
 
 /* Smallest m_batch served by the matrix-core kernels instead of the VALU kernel.  0 restores the
- * built-in rule (from 5 rows; from 3 rows on matrices of more than 256 16-row tiles, n_out > 4096; from 4 rows
- * on more than 128 tiles with 16 or more k steps;
- * from 2 rows on 1536 or more tiles with 8 or more k steps or more than 16384 units; int8 weights: from 5 rows,
- * from 3 rows on 1536 or more tiles; never for a single row); 17 keeps every batch size on the VALU kernel.  For tuning and tests.  Process-wide. */
+ * built-in rules: the k-stationary kernel (MGEMV_MATRIX_CORE_K_STATIONARY below) at 2-8 rows on int4 fp16 problems of
+ * 4-16 k steps of 512 whose 16-row tiles outnumber the compute units -- always with up to 8 k steps (2 rows: 8 k steps
+ * and 2.5 tiles per compute unit; 4-5 k steps: 1.5), with 9-16 where its walks of ceil(tiles / compute units) tiles fill
+ * the device better than the LDS-staged kernel's workgroups, or as well at 3-4 rows on walks of 2-3 or evenly divided
+ * tiles, at 5-8 rows up to 12 k steps on walks of 2, at 2 rows from walks of 3 --; else the LDS-staged (a single tile:
+ * the register-operand) kernel from 5 rows; from 3 rows on matrices of more than 256 tiles (n_out > 4096); from 4 rows
+ * on more than 128 tiles with 16 or more k steps; from 2 rows on 1536 or more tiles with 8 or more k steps or more than
+ * 16384 units; int8 weights: from 5 rows, from 3 rows on 1536 or more tiles; never for a single row.  17 keeps every
+ * batch size on the VALU kernel, 1 sends every batch size to the matrix cores.  For tuning and tests.  Process-wide. */
 MGEMV_API int mgemv_set_matrix_core_threshold(int min_m_batch);
 
 /* Which of the matrix-core kernels serves the small batches:
- *   MGEMV_MATRIX_CORE_AUTO (default)          the LDS-staged kernel wherever the matrix has at least two
- *                                             16-row tiles, else the register-operand kernel;
+ *   MGEMV_MATRIX_CORE_AUTO (default)          the k-stationary kernel where the built-in rule finds it ahead
+ *                                             (mgemv_set_matrix_core_threshold), else the LDS-staged kernel wherever
+ *                                             the matrix has at least two 16-row tiles, else the register-operand
+ *                                             kernel;
  *   MGEMV_MATRIX_CORE_REGISTER_OPERAND        always the kernel that reads its activation operand from
  *                                             L2 into registers;
  *   MGEMV_MATRIX_CORE_LDS_STAGED              the LDS-staged kernel wherever the matrix has at least two

@@ -284,16 +284,17 @@ inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
 //     10.34 / 10.37; 16384x8192 14.79 / 15.36; but 13312x8192 14.99 / 14.63, 13824x5120 10.97 / 10.60), at 5-8 rows
 //     only up to 12 k steps with walks of 2 (8192x6144 7.80 / 8.64; but 8192x8192 11.01 / 10.50, 16384x8192 16.42 /
 //     15.95, 14336x8192 16.0 / 15.3), at 2 rows from walks of 3 (12288x8192 12.74 / 13.28; 8192x8192 9.93 / 9.05);
-//   1 row: only with 9-16 k steps and walks from 7 tiles -- 28672x8192 22.2 / 22.5 (three leases: 1.9, 1.8, 0.5 %
-//     ahead), 32768x8192 25.5 / 26.9, 57344x8192 40.0 / 43.9 -- below that the VALU kernel's finer pipeline wins
-//     (16384x8192 14.9 / 13.1; 128256x4096, 8 waves, 47.8 / 45.7);
+//   1 row: never by this rule -- the single-row path is the VALU kernel by design.  Forced (threshold 1, this
+//     variant) it is ahead only with 9-16 k steps and even walks of 7 tiles or more: 28672x8192 22.2 / 22.5 (three
+//     leases: 1.9, 1.8, 0.5 % ahead), 32768x8192 25.5 / 26.9, 57344x8192 40.0 / 43.9; below that the VALU kernel's
+//     finer pipeline wins (16384x8192 14.9 / 13.1; 128256x4096, 8 waves, 47.8 / 45.7);
 //   9-16 rows: the operand takes two rounds through LDS and twice the registers' worth of L2 traffic per wave;
 //     level with the LDS-staged kernel or behind it (28672x8192 25.4 / 26.4; 28672x4096 16.0 / 15.2), left to it.
 inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int cus) {
   if (bits != 4 || m_batch > 8 || ksteps < 4) return false;
   const int walk = ceil_div(tiles, cus);
   const long long slots = (long long)walk * cus;  // tiles the launch has room for
-  if (m_batch == 1) return ksteps > 8 && walk >= 7 && slots * 100 <= (long long)tiles * 105;
+  if (m_batch == 1) return false;  // a single row stays on the VALU kernel, whatever was measured (above)
   if (ksteps <= 8) {
     if (m_batch == 2) return ksteps == 8 && tiles * 2 >= cus * 5;  // the VALU kernel's two rows are cheap: 8192x4096 5.90 / 5.95
     return ksteps <= 5 ? tiles * 2 >= cus * 3 : tiles > cus;

@@ -411,10 +411,8 @@ def test_adaptor_mirror_rejects_small_groups_like_the_reference():
 # test pins the rules, so a change to plan_launch that moves one of them shows up here.
 BUILTIN_PLANS = [
     # exact fit: one 4-wave workgroup per compute unit, every wave walking 7 tiles
-    ((28672, 1, 4096), dict(matrix_core=0, workgroups=256, threads=256, split_k=4, tiles_in_sequence=7)),
-    # ... and with 9-16 k steps and walks of 7 tiles or more, the k-stationary matrix-core kernel: one wave per k step
-    ((28672, 1, 8192), dict(matrix_core=3, workgroups=256, threads=1024, split_k=16, steps_per_wave=1, tiles_in_sequence=7)),
-    ((16384, 1, 8192), dict(matrix_core=0, workgroups=256, tiles_per_wg=4)),                   # walks of 4: the VALU kernel
+    ((28672, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256, split_k=4, tiles_in_sequence=7)),
+    ((57344, 1, 8192), dict(matrix_core=0)),                   # a single row never goes to the matrix cores
     ((8192, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256)),
     # at most one workgroup per compute unit: four k-split waves
     ((4096, 1, 4096), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=2)),
@@ -542,7 +540,7 @@ def test_default_plan_table_is_the_shipped_json_and_applies_to_256_compute_units
     path = os.path.join(os.path.dirname(_lib.LIB_PATH), "..", "default_plans.json")
     with open(path) as f:
         table = json.load(f)
-    assert table["format"] == 1 and mg.default_plan_count() == len(table["plans"])   # (it may be empty)
+    assert table["format"] == 1 and mg.default_plan_count() == len(table["plans"]) >= 1
     kinds = {0: 0, 1: 0, 2: 1, 3: 2, 4: 3}   # MGEMV_KERNEL_* -> what query_launch reports as matrix_core
     for e in table["plans"]:
         key = (e["n_out"], e["m_batch"], e["k"], e["weight_bits"], e["group_size"])
