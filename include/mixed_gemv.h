@@ -247,8 +247,9 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
                                         int max_workgroups);
 
 /* Smallest m_batch served by the matrix-core kernels instead of the VALU kernel.  0 restores the
- * built-in rules: the k-stationary kernel (MGEMV_MATRIX_CORE_K_STATIONARY below) at 2-8 rows on int4 fp16 problems of
- * 4-16 k steps of 512 whose 16-row tiles outnumber the compute units -- always with up to 8 k steps (2 rows: 8 k steps
+ * built-in rules: the k-stationary kernel (MGEMV_MATRIX_CORE_K_STATIONARY below) at 2-8 rows on fp16 problems of 4-16 k
+ * steps of 512 (int4; int8: 8-16 k steps of 256, which then count as "up to 8" here) whose 16-row tiles outnumber the
+ * compute units -- always with up to 8 k steps (2 rows: 8 k steps
  * and 2.5 tiles per compute unit; 4-5 k steps: 1.5), with 9-16 where its walks of ceil(tiles / compute units) tiles fill
  * the device better than the LDS-staged kernel's workgroups, or as well at 3-4 rows on walks of 2-3 or evenly divided
  * tiles, at 5-8 rows up to 12 k steps on walks of 2, at 2 rows from walks of 3 --; else the LDS-staged (a single tile:

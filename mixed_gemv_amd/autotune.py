@@ -45,6 +45,10 @@ def candidate_plans(n_out, k, weight_bits, m_batch):
             for split_k in (2, 4, 8):
                 out.append(dict(kernel=api.KERNEL_MATRIX_CORE_REGISTER_OPERAND, split_k=split_k,
                                 tiles_per_wave=tiles_per_wave))
+    # one wave per k step, one workgroup per compute unit (or two) walking the tiles; where the kernel does not exist
+    # (more than 16 k steps, bf16) the library falls back to its usual choice and the duplicate is dropped later
+    for cap in (0, 512):
+        out.append(dict(kernel=api.KERNEL_MATRIX_CORE_K_STATIONARY, max_workgroups=cap))
     return out
 
 

@@ -265,7 +265,7 @@ inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
 }
 
 // Where the k-stationary matrix-core kernel (one wave per k step, one workgroup per compute unit walking
-// ceil(tiles / cus) tiles) is ahead of the others; int4 weights, fp16, 4 to 16 k steps, up to 8 rows.  Its waves hold
+// ceil(tiles / cus) tiles) is ahead of the others; fp16, 4 to 16 k steps, 2 to 8 rows (int4 unless noted).  Its waves hold
 // their activation operand in registers, so its loop has neither barriers nor LDS reads and costs the same at 1 to
 // 8 rows; what it pays is a fixed start (operand through LDS, 0.8-1.6 us) and end (one barrier, one combine), and a
 // tail: when the weight stream ends, every wave of a SIMD still has a unit to compute.  Measured against the
@@ -288,14 +288,19 @@ inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
 //     variant) it is ahead only with 9-16 k steps and even walks of 7 tiles or more: 28672x8192 22.2 / 22.5 (three
 //     leases: 1.9, 1.8, 0.5 % ahead), 32768x8192 25.5 / 26.9, 57344x8192 40.0 / 43.9; below that the VALU kernel's
 //     finer pipeline wins (16384x8192 14.9 / 13.1; 128256x4096, 8 waves, 47.8 / 45.7);
+//   int8 weights (a k step is 256 long, the operand 32 registers): ahead on every shape tried at 3-8 rows, 16 waves
+//     and walks of 2 included -- 8192x4096 3 / 8 rows 7.68 / 8.12, 8.18 / 9.02; 11008x4096 8 rows 10.02 / 11.76;
+//     14336x2048 4 rows 7.49 / 8.58; 16384x4096 6 rows 12.87 / 14.34; 28672x4096 8 rows 20.69 / 21.57 -- so the
+//     rule of up to 8 k steps serves 8-16 there (78 launches on 19 further shapes: median +7.9 %; with 4-6 k steps
+//     it is 5-7 % behind);
 //   9-16 rows: the operand takes two rounds through LDS and twice the registers' worth of L2 traffic per wave;
 //     level with the LDS-staged kernel or behind it (28672x8192 25.4 / 26.4; 28672x4096 16.0 / 15.2), left to it.
 inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int cus) {
-  if (bits != 4 || m_batch > 8 || ksteps < 4) return false;
+  if (m_batch == 1 || m_batch > 8 || ksteps < 4) return false;  // a single row stays on the VALU kernel, whatever was measured (above)
   const int walk = ceil_div(tiles, cus);
   const long long slots = (long long)walk * cus;  // tiles the launch has room for
-  if (m_batch == 1) return false;  // a single row stays on the VALU kernel, whatever was measured (above)
-  if (ksteps <= 8) {
+  if (bits == 8 && ksteps < 8) return false;  // 8192x1024 int8, 3 rows: 4.9 us against 4.6; 32768x1536: 10.9 / 10.3
+  if (ksteps <= 8 || bits == 8) {
     if (m_batch == 2) return ksteps == 8 && tiles * 2 >= cus * 5;  // the VALU kernel's two rows are cheap: 8192x4096 5.90 / 5.95
     return ksteps <= 5 ? tiles * 2 >= cus * 3 : tiles > cus;
   }

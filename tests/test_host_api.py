@@ -532,6 +532,9 @@ def test_int8_weights_keep_two_to_four_rows_on_the_valu_kernel():
     assert [q(8192, m, 8192) for m in (2, 3, 4, 5)] == [0, 0, 0, 2]
     assert [q(4096, m, 11008) for m in (3, 4, 5)] == [0, 0, 2]
     assert [q(28672, m, 8192) for m in (2, 3, 4)] == [0, 2, 2]
+    # ... unless the k-stationary kernel takes the launch: 8-16 k steps of 256, 3-8 rows, more tiles than compute units
+    assert [q(8192, m, 4096) for m in (2, 3, 4, 8, 9)] == [0, 3, 3, 3, 2]
+    assert q(28672, 3, 4096) == 3 and q(28672, 2, 4096) == 0 and q(8192, 4, 1536) == 0 and q(4096, 8, 4096) == 2
 
 
 def test_default_plan_table_is_the_shipped_json_and_applies_to_256_compute_units_only():
