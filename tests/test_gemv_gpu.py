@@ -453,8 +453,8 @@ def test_each_activation_row_equals_the_single_row_result(gpu, m_batch):
 @pytest.mark.parametrize("bits,qop,g", [(4, SCALE_AND_ZEROS, 128), (4, SCALE_ONLY, 64), (4, PER_COLUMN, 0),
                                         (8, SCALE_AND_ZEROS, 64), (8, PER_COLUMN, 0), (4, SCALE_AND_ZEROS, 160)])
 def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
-    """The same batches through the two matrix-core kernels (LDS-staged at several k splits, register
-    operand) and the VALU kernel (threshold forced), ragged shape, every mode."""
+    """The same batches through the three matrix-core kernels (LDS-staged at several k splits, register
+    operand, k-stationary) and the VALU kernel (threshold forced), ragged shape, every mode."""
     n_out, k = 100, 1120 if g in (0, 160) else 1024
     for m_batch in (1, 5, 8, 13, 16):
         prob = Problem(f"mc{bits}{qop}", n_out, k, bits, qop, g, m_batch=m_batch, bias=True)
@@ -468,11 +468,12 @@ def test_matrix_core_and_valu_kernels_agree(gpu, bits, qop, g):
             for variant, split, tw in ((mg.MATRIX_CORE_LDS_STAGED, 0, 0), (mg.MATRIX_CORE_LDS_STAGED, 1, 2),
                                        (mg.MATRIX_CORE_LDS_STAGED, 2, 2), (mg.MATRIX_CORE_LDS_STAGED, 4, 1),
                                        (mg.MATRIX_CORE_LDS_STAGED, 2, 4), (mg.MATRIX_CORE_LDS_STAGED, 1, 8),
-                                       (mg.MATRIX_CORE_REGISTER_OPERAND, 0, 0)):
+                                       (mg.MATRIX_CORE_REGISTER_OPERAND, 0, 0), (mg.MATRIX_CORE_K_STATIONARY, 0, 0)):
                 mg.set_matrix_core_variant(variant)
                 mg.set_launch_override(split, tw, 0, 0)
                 plan = mg.query_launch(n_out, m_batch, k, bits)
-                assert plan["matrix_core"] == (2 if variant == mg.MATRIX_CORE_LDS_STAGED else 1)
+                assert plan["matrix_core"] == {mg.MATRIX_CORE_LDS_STAGED: 2, mg.MATRIX_CORE_REGISTER_OPERAND: 1,
+                                               mg.MATRIX_CORE_K_STATIONARY: 3}[variant]
                 if variant == mg.MATRIX_CORE_LDS_STAGED and tw and (8 if m_batch <= 8 else 16) // tw >= 2:
                     assert plan["tiles_per_wg"] == tw, plan
                 results.append(dev.run().copy())
