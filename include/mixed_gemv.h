@@ -247,12 +247,14 @@ MGEMV_API int mgemv_set_launch_override(int split_k_waves, int tiles_per_workgro
                                         int max_workgroups);
 
 /* Smallest m_batch served by the matrix-core kernels instead of the VALU kernel.  0 restores the
- * built-in rules: the k-stationary kernel (MGEMV_MATRIX_CORE_K_STATIONARY below) at 2-8 rows on fp16 problems of 4-16 k
+ * built-in rules: the k-stationary kernel (MGEMV_MATRIX_CORE_K_STATIONARY below) at 2-16 rows on fp16 problems of 4-16 k
  * steps of 512 (int4; int8: 8-16 k steps of 256, which then count as "up to 8" here) whose 16-row tiles outnumber the
  * compute units -- always with up to 8 k steps (2 rows: 8 k steps
  * and 2.5 tiles per compute unit; 4-5 k steps: 1.5), with 9-16 where its walks of ceil(tiles / compute units) tiles fill
  * the device better than the LDS-staged kernel's workgroups, or as well at 3-4 rows on walks of 2-3 or evenly divided
- * tiles, at 5-8 rows up to 12 k steps on walks of 2, at 2 rows from walks of 3 --; else the LDS-staged (a single tile:
+ * tiles, at 5-8 rows up to 12 k steps on walks of 2, at 2 rows from walks of 3; at 9-16 rows (int4) only where it fills
+ * the device better, the partial sums of a walk fit 128 KiB of LDS, and walks of 8-wave workgroups stay within 6 tiles
+ * --; else the LDS-staged (a single tile:
  * the register-operand) kernel from 5 rows; from 3 rows on matrices of more than 256 tiles (n_out > 4096); from 4 rows
  * on more than 128 tiles with 16 or more k steps; from 2 rows on 1536 or more tiles with 8 or more k steps or more than
  * 16384 units; int8 weights: from 5 rows, from 3 rows on 1536 or more tiles; never for a single row.  17 keeps every

@@ -265,7 +265,7 @@ inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
 }
 
 // Where the k-stationary matrix-core kernel (one wave per k step, one workgroup per compute unit walking
-// ceil(tiles / cus) tiles) is ahead of the others; fp16, 4 to 16 k steps, 2 to 8 rows (int4 unless noted).  Its waves hold
+// ceil(tiles / cus) tiles) is ahead of the others; fp16, 4 to 16 k steps, 2 to 16 rows (int4 unless noted).  Its waves hold
 // their activation operand in registers, so its loop has neither barriers nor LDS reads and costs the same at 1 to
 // 8 rows; what it pays is a fixed start (operand through LDS, 0.8-1.6 us) and end (one barrier, one combine), and a
 // tail: when the weight stream ends, every wave of a SIMD still has a unit to compute.  Measured against the
@@ -293,12 +293,26 @@ inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
 //     14336x2048 4 rows 7.49 / 8.58; 16384x4096 6 rows 12.87 / 14.34; 28672x4096 8 rows 20.69 / 21.57 -- so the
 //     rule of up to 8 k steps serves 8-16 there (78 launches on 19 further shapes: median +7.9 %; with 4-6 k steps
 //     it is 5-7 % behind);
-//   9-16 rows: the operand takes two rounds through LDS and twice the registers' worth of L2 traffic per wave;
-//     level with the LDS-staged kernel or behind it (28672x8192 25.4 / 26.4; 28672x4096 16.0 / 15.2), left to it.
+//   9-16 rows: the operand takes two rounds through LDS and twice the registers' worth of L2 traffic per wave, and
+//     the LDS-staged kernel shares a stage between up to 8 tiles there.  Ahead where that kernel's workgroups fill
+//     the machine worse by a tenth or more -- 11008x4096 16 rows 8.99 / 9.92; 10240x4096 8.68 / 9.87; 17408x4096
+//     12.59 / 14.40; 12288x8192 12 rows 15.04 / 16.31; 18432x8192 16 rows 20.56 / 25.39; 20480x8192 20.99 / 25.48;
+//     28672x8192 12 / 16 rows 25.75 / 27.08, 26.32 / 27.73 -- except on long walks of 8-wave workgroups (28672x4096
+//     12 rows 15.34 / 14.87; 22016x4096, walks of 6, 13.68 / 13.98 still ahead); level or behind where the two fill
+//     it alike (8192x6144 16 rows 10.44 / 9.90; 14336x8192 18.1 / 17.0; 14336x4096 12 rows 10.18 / 10.16) or where
+//     the partial sums of a walk do not fit the LDS and the workgroups double (32768x8192 35.1 / 30.0).
 inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int cus) {
-  if (m_batch == 1 || m_batch > 8 || ksteps < 4) return false;  // a single row stays on the VALU kernel, whatever was measured (above)
+  if (m_batch == 1 || ksteps < 4) return false;  // a single row stays on the VALU kernel, whatever was measured (above)
   const int walk = ceil_div(tiles, cus);
   const long long slots = (long long)walk * cus;  // tiles the launch has room for
+  if (m_batch > 8) {
+    // 9-16 rows: only where it fills the machine better than the LDS-staged kernel's workgroups of up to 8 tiles,
+    // the partial sums of a whole walk fit the LDS, and -- with up to 8 k steps, 2 waves per SIMD -- walks stay short
+    const int tw16 = lds_staged_tiles_per_wg(tiles, 16, cus);
+    const long long lds_slots16 = (long long)ceil_div(ceil_div(tiles, tw16), cus) * cus * tw16;
+    const long long park = (long long)walk * kKSlices * m_batch * kKStationaryParkSlots * 16;
+    return bits == 4 && lds_slots16 * 10 >= slots * 11 && park <= kMaxKStationaryLds && (ksteps > 8 || walk <= 6);
+  }
   if (bits == 8 && ksteps < 8) return false;  // 8192x1024 int8, 3 rows: 4.9 us against 4.6; 32768x1536: 10.9 / 10.3
   if (ksteps <= 8 || bits == 8) {
     if (m_batch == 2) return ksteps == 8 && tiles * 2 >= cus * 5;  // the VALU kernel's two rows are cheap: 8192x4096 5.90 / 5.95

@@ -472,13 +472,20 @@ BUILTIN_PLANS = [
     ((6144, 2, 4096), dict(matrix_core=0)),
     ((4608, 4, 2048), dict(matrix_core=0)),                    # 4 k steps: from 1.5 tiles per compute unit
     ((32768, 4, 1024), dict(matrix_core=2)),                   # 2 k steps, 2 waves per compute unit: no
-    ((28672, 9, 8192), dict(matrix_core=2)),                   # 9 rows and more: no
+    # 9-16 rows: only where it fills the machine better than the LDS-staged kernel's workgroups of up to 8 tiles and the
+    # partial sums of a walk fit the LDS; with up to 8 k steps only on walks of up to 6 tiles
+    ((28672, 9, 8192), dict(matrix_core=3, workgroups=256, tiles_in_sequence=7)),
+    ((28672, 16, 8192), dict(matrix_core=3, workgroups=256, tiles_in_sequence=7)),
+    ((11008, 16, 4096), dict(matrix_core=3, tiles_in_sequence=3)),
+    ((28672, 16, 4096), dict(matrix_core=2)),
+    ((32768, 16, 8192), dict(matrix_core=2)),
+    ((8192, 16, 6144), dict(matrix_core=2)),
     ((128256, 8, 4096), dict(matrix_core=3, workgroups=1024, tiles_in_sequence=8)),   # the partial sums of a walk must fit the LDS
     # tiles that share an activation stage: as few as give at most 256 workgroups ...
     ((5120, 8, 5120), dict(matrix_core=2, tiles_per_wg=2, workgroups=160, split_k=2, steps_per_wave=5, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((8192, 16, 8192), dict(matrix_core=2, tiles_per_wg=2, workgroups=256, split_k=4)),
     ((10240, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=160, variant=mg.MATRIX_CORE_LDS_STAGED)),
-    ((28672, 16, 8192), dict(matrix_core=2, tiles_per_wg=8, workgroups=224, split_k=1)),
+    ((28672, 16, 8192), dict(matrix_core=2, tiles_per_wg=8, workgroups=224, split_k=1, variant=mg.MATRIX_CORE_LDS_STAGED)),
     # ... or, when that cannot be had, a count whose last round of 256 is well filled
     ((28672, 8, 8192), dict(matrix_core=2, tiles_per_wg=4, workgroups=448, variant=mg.MATRIX_CORE_LDS_STAGED)),
     ((18944, 8, 3584), dict(matrix_core=2, tiles_per_wg=2, workgroups=592, split_k=1, variant=mg.MATRIX_CORE_LDS_STAGED)),

@@ -158,7 +158,7 @@ def test_the_built_in_rule_takes_it_where_it_was_measured_ahead(gpu):
         assert rel <= REL_TOL, (rows, k, rel)
     n_out = 16 * 2 * cus
     assert mg.query_launch(n_out, 2, 4096, 4, 128, num_compute_units=cus)["matrix_core"] == 0     # 2 rows on walks of 2: VALU
-    assert mg.query_launch(n_out, 16, 4096, 4, 128, num_compute_units=cus)["matrix_core"] == 2    # 9-16 rows: LDS-staged
+    assert mg.query_launch(n_out, 16, 4096, 4, 128, num_compute_units=cus)["matrix_core"] == 2    # 9-16 rows, filled alike: LDS-staged
     assert mg.query_launch(n_out, 4, 1024, 4, 128, num_compute_units=cus)["matrix_core"] != 3      # 2 k steps: too few waves
     assert mg.query_launch(n_out, 4, 16384, 4, 128, num_compute_units=cus)["matrix_core"] == 2     # 32 k steps: no such launch
     assert mg.query_launch(n_out, 4, 4096, 4, 128, element="bf16", num_compute_units=cus)["matrix_core"] == 2   # fp16 only
