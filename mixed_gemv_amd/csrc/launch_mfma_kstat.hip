@@ -13,14 +13,17 @@ namespace mgemv {
 // blockDim = 64 * ksteps (at most 16 waves): wave kw of a workgroup owns k step kw of EVERY tile
 // the workgroup walks.  The activation operand of a k step -- x[batch row lane % 16][the lane's 8 k
 // of each of the 16 matrix instructions], 64 registers for int4 -- therefore never changes: it is
-// loaded once, in front of the walk, and the loop over the tiles
-// holds nothing but the weight stream (one unit of 4 KiB per wave and tile, the next tile's unit in
-// flight while one is computed), the dequantiser and sixteen matrix instructions.  No LDS stage, no
-// barrier and no activation traffic inside the loop; a wave's partial products of a tile (a 16 x 16
-// fp32 block, of which m_batch columns matter) are parked in LDS, and after the walk one barrier
-// separates the walks from the combine: wave r sums the ksteps partial blocks of tiles r, r + waves,
-// ... and stores them.  Per eight int4 weights a lane issues 13 VALU instructions and one matrix
+// loaded once, in front of the walk, and the loop over the tiles holds nothing but the weight
+// stream (one unit of 4 KiB per wave and tile, the next tile's unit in flight while one is
+// computed), the dequantiser and sixteen matrix instructions.  No LDS stage, no barrier and no
+// activation traffic inside the loop; a wave's partial products of a tile (a 16 x 16 fp32 block, of
+// which m_batch columns matter) are parked in LDS, and after the walk one barrier separates the
+// walks from the combine: wave r sums the ksteps partial blocks of tiles r, r + waves, ... and
+// stores them.  Per eight int4 weights a lane issues 13 VALU instructions and one matrix
 // instruction, against 17 VALU instructions of the DPP-dot kernel, whatever the number of rows.
+// It replaces nothing in the reference, whose kernel is fixed to one activation row
+// (gemv/threadblock/default_mma_core_simt.h:68-70); the dequantiser is the one of every kernel here
+// (gemv/warp/warp_dequantizer.h:52-59, 86-92), the epilogue host/mixed_gemv.h:102-103.
 // Dynamic LDS: waves x 8 activation rows (the stage each wave turns its operand round in, at the start) and
 // tiles of the longest walk x 4 x m_batch x 17 x 16 bytes (the partial sums) -- one behind the other where
 // both fit, else sharing the space, with a barrier between the two uses.
@@ -110,9 +113,9 @@ gemv_mfma_kstat_kernel(const uint8_t* weights, const half_t* x, const half_t* sc
   // once, where a real one would have to land before the combine may reuse its register.
   auto offsets_of_tile = [&](int i, int (&off)[GROUPS_PER_RUN]) {
     const int row = (tile0 + i) * kTileRows + m;
-    const int row_bytes = (row < p.n_out ? row : p.n_out - 1) * 2 + (i < my_tiles ? 0 : 0x40000000);
+    const uint32_t row_bytes = (uint32_t)(row < p.n_out ? row : p.n_out - 1) * 2u + (i < my_tiles ? 0u : 0x40000000u);
 #pragma unroll
-    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) off[gi] = group_offset[gi] + row_bytes;
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) off[gi] = (int)((uint32_t)group_offset[gi] + row_bytes);
   };
 
   MfmaActivations<BITS> xa;
