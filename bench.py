@@ -543,18 +543,23 @@ def ceilings_of_rows(wl, use_graph):
     import torch
     import mixed_gemv_amd as mg
     plan = mg.query_launch(wl.n_out, wl.m_batch, wl.k, 4, wl.group)
-    if wl.bits != 4 or wl.quant_op != 3 or plan["matrix_core"] != 2 or plan["tiles_per_wg"] < 2:
+    kstat = plan["matrix_core"] == 3
+    if wl.bits != 4 or wl.quant_op != 3 or not (kstat or (plan["matrix_core"] == 2 and plan["tiles_per_wg"] >= 2)):
         return None
     w_bytes = wl.w[0].numel()
     sink = torch.zeros(1, dtype=torch.int32, device=wl.y.device)
     waves = plan["threads"] // 64
     out = {"weight_bytes": w_bytes, "algorithmic_bytes": wl.bytes,
-           "launch": {k: plan[k] for k in ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave")}}
+           "kernel": "k-stationary matrix-core kernel" if kstat else "LDS-staged matrix-core kernel",
+           "launch": {k: plan[k] for k in ("workgroups", "threads", "split_k", "tiles_per_wg", "steps_per_wave", "tiles_in_sequence")}}
     probe = _Launches(lambda i: mg.probe_stream_read(wl.w[i % wl.sets], w_bytes, plan["workgroups"], waves, 2, sink), wl.sets)
     _, ev_us, *_ = time_workload(probe, 300, 20, use_graph=use_graph, repetitions=5)
     out["stream_read"] = {"us_per_launch": round(ev_us, 3), "note": "plain streaming read of the weight bytes, the launch's shape"}
-    for key, kind, note in (("loads_only", mg.PROBE_LOADS_ONLY, "every load, the staging of the activation rows and the barriers; no arithmetic"),
-                            ("compute_only", mg.PROBE_COMPUTE_ONLY, "only the first k step of each wave loaded; its staging and arithmetic repeated per k step")):
+    notes = (("every load, the operand's way through LDS, the parking of the partial sums, the barrier and the combine; no arithmetic",
+              "only the first tile's unit of each wave loaded; its arithmetic repeated for every tile of the walk") if kstat else
+             ("every load, the staging of the activation rows and the barriers; no arithmetic",
+              "only the first k step of each wave loaded; its staging and arithmetic repeated per k step"))
+    for key, kind, note in (("loads_only", mg.PROBE_LOADS_ONLY, notes[0]), ("compute_only", mg.PROBE_COMPUTE_ONLY, notes[1])):
         probe = _Launches(lambda i, kind=kind: mg.probe_gemv_rows(kind, wl.m_batch, wl.w[i % wl.sets], wl.x, wl.s[i % wl.sets],
                                                                   wl.z[i % wl.sets], wl.y, wl.n_out, wl.k, wl.group), wl.sets)
         _, ev_us, *_ = time_workload(probe, 300, 20, use_graph=use_graph, repetitions=5)
@@ -845,7 +850,7 @@ def main():
             entry["parity"] = parity_summary(w2, sets, threads, with_dequant=(rows in (None, 1)))
         if base == "c5" and rows is None and element == "f16" and batch == 1 and not args.no_ceilings:
             out.setdefault("ceilings", {})[base] = ceilings_of(w2, use_graph, timeline=True)
-        if base == "c4" and rows in (8, 16) and element == "f16" and batch == 1 and not args.no_ceilings:
+        if ((base == "c4" and rows in (8, 16)) or (base == "c5" and rows in (4, 16))) and element == "f16" and batch == 1 and not args.no_ceilings:
             c = ceilings_of_rows(w2, use_graph)
             if c is not None:
                 out.setdefault("ceilings", {})[name] = c

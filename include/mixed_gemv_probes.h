@@ -68,9 +68,13 @@ MGEMV_API int mgemv_probe_gemv(int kind, unsigned long long *trace, size_t trace
 /* The same two builds -- MGEMV_PROBE_LOADS_ONLY, MGEMV_PROBE_COMPUTE_ONLY -- for a launch of m_batch
  * activation rows, where they exist: one row as above; on the matrix cores the LDS-staged kernel whose
  * workgroups share their activation stage between two or more tiles (int4, scale and zero, fp16,
- * group sizes 64-512; e.g. 8192 x 8192 at 4-16 rows).  There "loads only" keeps the staging of the
+ * group sizes 64-512; e.g. 8192 x 8192 at 8-16 rows), and the k-stationary kernel (same operand types;
+ * e.g. 28672 x 8192 at 2-16 rows).  On the LDS-staged kernel "loads only" keeps the staging of the
  * activation rows and the barriers, and "compute only" requests a wave's first k step only and
- * repeats that step's staging and arithmetic.  Other launches return MGEMV_ERR_QUANT_OP. */
+ * repeats that step's staging and arithmetic; on the k-stationary kernel "loads only" keeps the
+ * operand's way through LDS, the parking of the partial sums, the barrier and the combine, and
+ * "compute only" requests the first tile's unit only and repeats its arithmetic for every tile of
+ * the walk.  Other launches return MGEMV_ERR_QUANT_OP. */
 MGEMV_API int mgemv_probe_gemv_rows(int kind, int m_batch, const void *weights, const uint16_t *x,
                                     const uint16_t *scale, const uint16_t *zero_add, uint16_t *y, int n_out, int k,
                                     int group_size, void *stream);

@@ -716,10 +716,13 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
     g.tail.m_batch = m_batch;
     g.lds = launch_resources(g.plan, weight_bits, m_batch, act).lds_bytes;
     if (g.plan.k_stationary) {
-      if (probe != kProbeNone) return MGEMV_ERR_QUANT_OP;  // no measurement builds of this kernel
       const size_t stage = (size_t)g.plan.split_k * 8 * (step_k(weight_bits) * 2 + 16);
       if (g.lds > stage && g.lds - stage >= (size_t)g.plan.tiles_in_sequence * kKSlices * m_batch * kKStationaryParkSlots * 16)
         g.tail.flags |= kParkBehindStage;
+      if (probe != kProbeNone) {
+        if (probe == kProbeTimeline || !mfma_kstat_probe_exists(weight_bits, quant_op, gpr, act)) return MGEMV_ERR_QUANT_OP;
+        return launch_mfma_kstat_probe(g, gpr, probe) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
+      }
       return launch_mfma_kstat(g, weight_bits, quant_op, gpr, act) == hipSuccess ? MGEMV_OK : MGEMV_ERR_LAUNCH;
     }
     if (probe != kProbeNone) {

@@ -265,6 +265,9 @@ hipError_t launch_gemv_bf16(const GemvLaunch& g, int bits, int qop, int mb, int 
 hipError_t launch_mfma(const GemvLaunch& g, int bits, int qop, int gpr);
 hipError_t launch_mfma_lds(const GemvLaunch& g, int bits, int qop, int gpr, int rounds, int act);
 hipError_t launch_mfma_kstat(const GemvLaunch& g, int bits, int qop, int gpr, int act);
+// ... and of the k-stationary matrix-core kernel (kProbeLoadsOnly / kProbeComputeOnly), where they exist.
+bool mfma_kstat_probe_exists(int bits, int qop, int gpr, int act);
+hipError_t launch_mfma_kstat_probe(const GemvLaunch& g, int gpr, int probe);
 // Measurement builds of the single-row int4 scale-and-zero fp16 VALU kernel (probe: kProbeLoadsOnly / kProbeTimeline / kProbeComputeOnly).
 hipError_t launch_gemv_probe(const GemvLaunch& g, int probe);
 // ... and of the LDS-staged matrix-core kernel (kProbeLoadsOnly / kProbeComputeOnly), where they exist.

@@ -44,7 +44,10 @@ __device__ __forceinline__ void load_unit_kstat(MfmaWeights<BITS, GROUPS_PER_RUN
   }
 }
 
-template <int BITS, int QOP, int GROUPS_PER_RUN, int ACT>
+// PROBE (measurement builds, wrong results): kProbeLoadsOnly keeps every load, the operand's way through LDS, the
+// parking, the barrier and the combine, and replaces the arithmetic of a unit by taking its registers;
+// kProbeComputeOnly requests only the first tile's unit and repeats its arithmetic for every tile of the walk.
+template <int BITS, int QOP, int GROUPS_PER_RUN, int ACT, int PROBE = kProbeNone>
 __global__ void __launch_bounds__(kWave * kMaxWavesPerWorkgroup)
 gemv_mfma_kstat_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, const half_t* zero_add, int n_out,
                        int k, uint32_t packed_steps, int workgroups, int num_groups, uint32_t packed_group,
@@ -181,13 +184,32 @@ gemv_mfma_kstat_kernel(const uint8_t* weights, const half_t* x, const half_t* sc
       const uint32_t bits[1] = {f.s[0]};
       short_ok = short_ok && wave_scales_permit_short_form<ACT>(bits);
     }
-    compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, f, xa, c, col_scale, short_ok);
+    if constexpr (PROBE == kProbeLoadsOnly) {
+      uint32_t t = xa.x[0][0][0];
+#pragma unroll
+      for (int b = 0; b < kBlocksPerUnit; ++b) t ^= f.w[b][0] ^ f.w[b][1] ^ f.w[b][2] ^ f.w[b][3];
+#pragma unroll
+      for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) t ^= f.s[gi] ^ f.z[gi];
+      acc[0] += __builtin_bit_cast(float, t & 0x3fffffffu);
+    } else {
+      compute_unit_mfma<BITS, QOP, GROUPS_PER_RUN, ACT>(acc, f, xa, c, col_scale, short_ok);
+    }
     if (m < m_batch) my_park[i * park_tile_stride] = acc;
+  };
+  // arithmetic-only build: the next unit is the first one again; the compiler must assume its registers changed
+  auto repeat_first_unit = [&](MfmaWeights<BITS, GROUPS_PER_RUN>& to, const MfmaWeights<BITS, GROUPS_PER_RUN>& from) {
+    to = from;
+#pragma unroll
+    for (int b = 0; b < kBlocksPerUnit; ++b) asm volatile("" : "+v"(to.w[b]));
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_RUN; ++gi) asm volatile("" : "+v"(to.s[gi]), "+v"(to.z[gi]));
   };
 
   int i = 0;
   do {
-    {
+    if constexpr (PROBE == kProbeComputeOnly) {
+      repeat_first_unit(wb, wa);
+    } else {
       int off[GROUPS_PER_RUN];
       offsets_of_tile(i + 1, off);
       load_unit_kstat<BITS, QOP, GROUPS_PER_RUN>(wb, w_rsrc, tables, (i + 1) * tile_stride + lane * kChunkBytes, off);
@@ -195,7 +217,9 @@ gemv_mfma_kstat_kernel(const uint8_t* weights, const half_t* x, const half_t* sc
     __builtin_amdgcn_sched_barrier(0);
     compute_and_park(wa, i);
     __builtin_amdgcn_sched_barrier(0);
-    {
+    if constexpr (PROBE == kProbeComputeOnly) {
+      repeat_first_unit(wa, wb);
+    } else {
       int off[GROUPS_PER_RUN];
       offsets_of_tile(i + 2, off);
       load_unit_kstat<BITS, QOP, GROUPS_PER_RUN>(wa, w_rsrc, tables, (i + 2) * tile_stride + lane * kChunkBytes, off);
@@ -276,9 +300,9 @@ gemv_mfma_kstat_kernel(const uint8_t* weights, const half_t* x, const half_t* sc
   }
 }
 
-template <int BITS, int QOP, int GPR, int ACT>
+template <int BITS, int QOP, int GPR, int ACT, int PROBE = kProbeNone>
 hipError_t launch_mfma_kstat_kernel(const GemvLaunch& g) {
-  const auto kernel = gemv_mfma_kstat_kernel<BITS, QOP, GPR, ACT>;
+  const auto kernel = gemv_mfma_kstat_kernel<BITS, QOP, GPR, ACT, PROBE>;
   if (g.lds > 48 * 1024) {
     // More than 48 KiB of dynamic LDS has to be granted per kernel and device; remember the
     // largest grant so that only the first such launch pays for the call.
@@ -329,6 +353,20 @@ hipError_t launch_mfma_kstat_act(const GemvLaunch& g, int bits, int qop, int gpr
     case 2: return launch_mfma_kstat_gpr<8, 2, ACT>(g, gpr);
     default: return launch_mfma_kstat_gpr<8, 3, ACT>(g, gpr);
   }
+}
+
+// Measurement builds exist for int4 scale-and-zero fp16 launches with one or two groups per lane run.
+bool mfma_kstat_probe_exists(int bits, int qop, int gpr, int act) {
+  return bits == 4 && qop == MGEMV_FINEGRAINED_SCALE_AND_ZEROS && (gpr == 1 || gpr == 2) && act == kActF16;
+}
+
+hipError_t launch_mfma_kstat_probe(const GemvLaunch& g, int gpr, int probe) {
+  constexpr int kQ = MGEMV_FINEGRAINED_SCALE_AND_ZEROS;
+  if (probe == kProbeLoadsOnly)
+    return gpr == 1 ? launch_mfma_kstat_kernel<4, kQ, 1, kActF16, kProbeLoadsOnly>(g)
+                    : launch_mfma_kstat_kernel<4, kQ, 2, kActF16, kProbeLoadsOnly>(g);
+  return gpr == 1 ? launch_mfma_kstat_kernel<4, kQ, 1, kActF16, kProbeComputeOnly>(g)
+                  : launch_mfma_kstat_kernel<4, kQ, 2, kActF16, kProbeComputeOnly>(g);
 }
 
 hipError_t launch_mfma_kstat(const GemvLaunch& g, int bits, int qop, int gpr, int act) {

@@ -164,13 +164,33 @@ def test_the_built_in_rule_takes_it_where_it_was_measured_ahead(gpu):
     assert mg.query_launch(n_out, 4, 4096, 4, 128, element="bf16", num_compute_units=cus)["matrix_core"] == 2   # fp16 only
 
 
-def test_measurement_builds_are_refused(gpu):
+def test_measurement_builds(gpu):
+    """Arithmetic-only: with walks of one tile every unit is loaded, and the result is the product's, bit for bit.
+    Loads-only, and arithmetic-only on longer walks: they run and write every output.  No time-stamped build, and none
+    for group sizes that put four groups on a lane's run."""
     import torch
     from mixed_gemv_amd._lib import MixedGemvError
-    prob = Problem("ks_probe", 512, 4096, 4, SCALE_AND_ZEROS, 128)
+    prob = Problem("ks_probe", 512, 4096, 4, SCALE_AND_ZEROS, 128, m_batch=5, x_dist="normal")
     dev = DeviceProblem(prob, gpu)
     trace = torch.zeros((4096, mg.PROBE_TIMELINE_WORDS), dtype=torch.int64, device=gpu)
     with k_stationary(0):
-        for kind in (mg.PROBE_LOADS_ONLY, mg.PROBE_COMPUTE_ONLY, mg.PROBE_TIMELINE):
-            with pytest.raises(MixedGemvError):
-                mg.probe_gemv(kind, trace, dev.w, dev.x, dev.scale, dev.zero, dev.y, 512, 4096, 128)
+        assert mg.query_launch(512, 5, 4096, 4, 128)["tiles_in_sequence"] == 1
+        want = dev.run().copy()
+        dev.y.fill_(0x7e00)
+        mg.probe_gemv_rows(mg.PROBE_COMPUTE_ONLY, 5, dev.w, dev.x, dev.scale, dev.zero, dev.y, 512, 4096, 128)
+        torch.cuda.synchronize()
+        assert np.array_equal(dev.y.cpu().numpy().view(np.uint16), want.view(np.uint16))
+        dev.y.fill_(0x7e00)
+        mg.probe_gemv_rows(mg.PROBE_LOADS_ONLY, 5, dev.w, dev.x, dev.scale, dev.zero, dev.y, 512, 4096, 128)
+        torch.cuda.synchronize()
+        assert not np.any(dev.y.cpu().numpy().view(np.uint16) == 0x7e00)
+    with k_stationary(4):     # walks of 8 tiles: both builds run and write every output
+        for kind in (mg.PROBE_LOADS_ONLY, mg.PROBE_COMPUTE_ONLY):
+            dev.y.fill_(0x7e00)
+            mg.probe_gemv_rows(kind, 5, dev.w, dev.x, dev.scale, dev.zero, dev.y, 512, 4096, 128)
+            torch.cuda.synchronize()
+            assert not np.any(dev.y.cpu().numpy().view(np.uint16) == 0x7e00)
+        with pytest.raises(MixedGemvError):
+            mg.probe_gemv(mg.PROBE_TIMELINE, trace, dev.w, dev.x, dev.scale, dev.zero, dev.y, 512, 4096, 128)
+        with pytest.raises(MixedGemvError):     # group size 96: four groups per lane run, no measurement build
+            mg.probe_gemv_rows(mg.PROBE_LOADS_ONLY, 5, dev.w, dev.x, dev.scale, dev.zero, dev.y, 512, 768, 96)

@@ -94,9 +94,15 @@ def test_matrix_core_measurement_builds_run(gpu, m_batch):
             mg.probe_gemv_rows(mg.PROBE_TIMELINE, 8, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 64)
     finally:
         mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
-    if m_batch <= 8:
-        with pytest.raises(MixedGemvError):     # the k-stationary kernel has no measurement builds
-            mg.probe_gemv_rows(mg.PROBE_LOADS_ONLY, m_batch, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 64)
+    if m_batch <= 8:    # the built-in rule: the k-stationary kernel, whose measurement builds write every output too
+        assert mg.query_launch(n_out, m_batch, k, 4, 64)["matrix_core"] == 3
+        for kind in (mg.PROBE_LOADS_ONLY, mg.PROBE_COMPUTE_ONLY):
+            dev.y.fill_(0x7e00)
+            mg.probe_gemv_rows(kind, m_batch, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 64)
+            torch.cuda.synchronize()
+            assert not np.any(dev.y.cpu().numpy().view(np.uint16) == 0x7e00)
+        with pytest.raises(MixedGemvError):
+            mg.probe_gemv_rows(mg.PROBE_TIMELINE, m_batch, dev.w, dev.x, dev.scale, dev.zero, dev.y, n_out, k, 64)
 
 
 def test_stream_read_and_empty_launch_run_and_check_their_arguments(gpu):
