@@ -46,6 +46,9 @@ CASES = [
     ("k_not_a_multiple_of_the_step", 304, 1000, 4, PER_COLUMN, 0, 6, True, 8, (0.001, 0.02)),
     ("exact_integer_form", 528, 2048, 4, SCALE_AND_ZEROS, 128, 8, False, 8, (0.05, 0.3)),
     ("walks_of_7_like_28672x8192", 7 * 16 * 24, 8192, 4, SCALE_AND_ZEROS, 128, 4, False, 24, (0.001, 0.02)),
+    ("a_single_tile", 16, 8192, 4, SCALE_AND_ZEROS, 128, 8, True, 0, (0.001, 0.02)),
+    ("four_output_rows", 4, 512, 4, SCALE_AND_ZEROS, 64, 16, True, 0, (0.001, 0.02)),
+    ("one_k_step_of_8", 48, 8, 8, PER_COLUMN, 0, 3, False, 0, (0.001, 0.01)),
 ]
 
 
