@@ -164,6 +164,25 @@ MGEMV_API int mgemv_gemv_batched(const void *weights, const uint16_t *x, const u
                                  int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
                                  int64_t stride_bias, int64_t stride_y, void *stream);
 
+/* Routed launch over a stack of matrices -- the use that the 3-D, expert-stacked shapes of the
+ * reference's preprocessor are for (utils/preprocess.h:134-136, 315-317).  The reference has no
+ * such launch: its batch arguments step through a stack at a fixed stride
+ * (gemv/kernel/mixed_gemv.h:140-149), so a decode step that wants the top-k experts of a token
+ * would need one launch per expert.  As mgemv_gemv_batched, except that problem b takes the
+ * weights, scales, zeros and bias of entry route[b] of the stack (their strides are multiplied by
+ * route[b]), while x and y are still stepped by b (stride_x = 0: one token and its chosen
+ * experts).  route is a DEVICE array of batch_count 32-bit indices, read by the kernel, so a
+ * router's output is used where it lies, with no copy to the host; route_extent is the number of
+ * entries in the stack.  A problem whose index lies outside [0, route_extent) is skipped, its
+ * outputs are left as they were (the host cannot check device data without a synchronisation, and
+ * an unchecked index would be a read outside the stack).  Results are those of
+ * mgemv_gemv_batched on the same matrices, bit for bit. */
+MGEMV_API int mgemv_gemv_routed(const void *weights, const uint16_t *x, const uint16_t *scale,
+                                const uint16_t *zero_add, const uint16_t *bias, uint16_t *y, const int32_t *route,
+                                int route_extent, int batch_count, int n_out, int m_batch, int k, int group_size,
+                                int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x,
+                                int64_t stride_scale, int64_t stride_bias, int64_t stride_y, void *stream);
+
 /* GemvAdaptor::Arguments (gemv/device/gemv_adaptor.h:114-178) as a plain struct, and
  * GemvAdaptor::operator()(args, stream) (:258-261) as one call: everything mgemv_gemv_batched
  * takes, plus the epilogue's alpha and beta and the leading dimensions of the reference's
@@ -322,6 +341,12 @@ MGEMV_API int mgemv_gemv_batched_bf16(const void *weights, const uint16_t *x, co
                                       int n_out, int m_batch, int k, int group_size, int quant_op, int weight_bits,
                                       int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
                                       int64_t stride_bias, int64_t stride_y, void *stream);
+MGEMV_API int mgemv_gemv_routed_bf16(const void *weights, const uint16_t *x, const uint16_t *scale,
+                                     const uint16_t *zero_add, const uint16_t *bias, uint16_t *y,
+                                     const int32_t *route, int route_extent, int batch_count, int n_out, int m_batch,
+                                     int k, int group_size, int quant_op, int weight_bits, int64_t stride_weights,
+                                     int64_t stride_x, int64_t stride_scale, int64_t stride_bias, int64_t stride_y,
+                                     void *stream);
 MGEMV_API int mgemv_dequantize_bf16(const void *weights, const uint16_t *scale, const uint16_t *zero_add,
                                     uint16_t *out, int n_out, int k, int group_size, int quant_op, int weight_bits,
                                     void *stream);

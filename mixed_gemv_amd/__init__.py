@@ -14,6 +14,7 @@ from .api import (  # noqa: F401
     ZeroPointPreprocessor,
     dequantize,
     device_gemv,
+    device_gemv_routed,
     gemv_arguments,
     host_gemv,
     static_scratch_bytes_needed,

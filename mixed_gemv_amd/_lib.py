@@ -27,6 +27,10 @@ SIGNATURES = {
     "mgemv_gemv": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 6 + [_vp]),
     "mgemv_gemv_batched": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 7
                            + [_c.c_int64] * 5 + [_vp]),
+    "mgemv_gemv_routed": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p, _vp] + [_c.c_int] * 8
+                          + [_c.c_int64] * 5 + [_vp]),
+    "mgemv_gemv_routed_bf16": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p, _vp] + [_c.c_int] * 8
+                               + [_c.c_int64] * 5 + [_vp]),
     "mgemv_dequantize": (_c.c_int, [_vp, _u16p, _u16p, _u16p] + [_c.c_int] * 5 + [_vp]),
     "mgemv_gemv_bf16": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 6 + [_vp]),
     "mgemv_gemv_batched_bf16": (_c.c_int, [_vp, _u16p, _u16p, _u16p, _u16p, _u16p] + [_c.c_int] * 7

@@ -245,6 +245,22 @@ def device_gemv(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, B, M, N, 
     _lib.check(st, "device_gemv")
 
 
+def device_gemv_routed(ptr_A, ptr_B, ptr_scale, ptr_zero_point, ptr_C, ptr_D, route, stack_entries, B, M, N, K,
+                       group_size, batch_strides, quant_op=WeightOnlyQuantOp.FINEGRAINED_SCALE_AND_ZEROS,
+                       weight_bits=4, stream=None, element=None):
+    """device_gemv over an expert stack (the 3-D shapes of utils/preprocess.h:134-136), routed: problem
+    b of B takes the weights, scales, zeros and bias of entry route[b] (a DEVICE array of int32) of the
+    stack of stack_entries matrices; x and y are stepped by b.  batch_strides = (weights in bytes, x,
+    scale, bias, y) as in device_gemv; a stride of 0 for x gives every problem the same activations.
+    The reference steps through a stack at a fixed stride only (gemv/kernel/mixed_gemv.h:140-149)."""
+    fn = _lib.lib().mgemv_gemv_routed_bf16 if _is_bf16(element, ptr_B) else _lib.lib().mgemv_gemv_routed
+    sa, sb, ss, sc, sd = batch_strides
+    st = fn(_dev_ptr(ptr_A), _dev_ptr(ptr_B), _dev_ptr(ptr_scale), _dev_ptr(ptr_zero_point), _dev_ptr(ptr_C),
+            _dev_ptr(ptr_D), _dev_ptr(route), int(stack_entries), int(B), int(M), int(N), int(K), int(group_size),
+            int(quant_op), int(weight_bits), int(sa), int(sb), int(ss), int(sc), int(sd), _stream_ptr(stream))
+    _lib.check(st, "device_gemv_routed")
+
+
 class GemvAdaptor:
     """gemv/device/gemv_adaptor.h:114-261: Arguments / initialize / run / __call__."""
 

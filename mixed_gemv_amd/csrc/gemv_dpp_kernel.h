@@ -384,7 +384,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   p.workgroups = workgroups;
   p.wgs_per_xcd = (workgroups + kNumXcd - 1) / kNumXcd;
   p.group_size = (int)(packed_group & 0xffffffu);
-  p.tiles_per_wg = (int)(packed_group >> 24);
+  p.tiles_per_wg = tiles_per_wg_of(packed_group);
   // The library is built with kernel-argument preloading: the four pointers and six words in
   // front of GemvTail arrive in SGPRs with the wave (firmware without the feature runs a short
   // prologue that loads them instead).  Nothing on the way to the first weight loads of an
@@ -392,13 +392,20 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   // for any scalar load at all: `tail` itself is only touched by batched launches and tile
   // walks, everything else reads the copy `late`, fetched once the first unit is requested.
   // Batched launch (gemv/kernel/mixed_gemv.h:140-149, 222-223): problems past the first fetch
-  // their strides first.
+  // their strides first.  A routed launch (a bit of a preloaded word says so) looks up whose
+  // weights, scales, zeros and bias each problem takes; x and y stay with the problem.
   const long long batch = blockIdx.z;
-  if (batch != 0) {
-    p.weights += batch * tail.stride_weights;
+  long long owner = batch;
+  if ((blockIdx.z | (packed_group & kRoutedLaunch)) != 0) {  // one test on the way of an unbatched launch
+    if ((packed_group & kRoutedLaunch) != 0) {
+      const int entry = tail.route[batch];
+      if ((unsigned)entry >= (unsigned)tail.route_extent) return;  // whole workgroup, before any barrier
+      owner = entry;
+    }
+    p.weights += owner * tail.stride_weights;
     p.x += batch * tail.stride_x;
-    p.scale += batch * tail.stride_scale;
-    p.zero_add += batch * tail.stride_scale;  // only dereferenced in scale+zero mode
+    p.scale += owner * tail.stride_scale;
+    p.zero_add += owner * tail.stride_scale;  // only dereferenced in scale+zero mode
   }
 
   const int wg = logical_workgroup(p);
@@ -538,7 +545,7 @@ gemv_dpp_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, co
   const int split_k = late.split_k;
   const int park_stride = p.tiles_per_wg * split_k * MB * kWave;
   const bool has_bias = late.bias != nullptr;
-  late.bias += batch * late.stride_bias;
+  late.bias += owner * late.stride_bias;
   late.y += batch * late.stride_y;
 
   // Split-K combine (gemv/threadblock/accumulator_combine.h:269-329): every wave has parked
@@ -584,7 +591,7 @@ template <int BITS, int QOP, int MB, int GPR, bool MULTI, int ACT>
 hipError_t launch_gemv_kernel_m(const GemvLaunch& g) {
   return launch(gemv_dpp_kernel<BITS, QOP, MB, GPR, MULTI, ACT>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
                 g.zero_add, g.n_out, g.k, pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups,
-                g.tail.num_groups, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+                g.tail.num_groups, pack_group(g.group_size, g.plan.tiles_per_wg, g.tail.route != nullptr), g.tail);
 }
 
 template <int BITS, int QOP, int MB, int GPR, int ACT>

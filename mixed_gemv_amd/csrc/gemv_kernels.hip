@@ -664,8 +664,10 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
              int quant_op, int weight_bits, int64_t stride_weights, int64_t stride_x, int64_t stride_scale,
              int64_t stride_bias, int64_t stride_y, void* stream, int act, float alpha = 1.0f, float beta = 1.0f,
              int probe = kProbeNone, unsigned long long* trace = nullptr, size_t trace_capacity_waves = 0,
-             bool timed_waits = false) {
+             bool timed_waits = false, const int32_t* route = nullptr, int route_extent = 0) {
   if (batch_count < 1 || batch_count > 65535) return MGEMV_ERR_BATCH;
+  if (route != nullptr && route_extent < 1) return MGEMV_ERR_BATCH;
+  if (reinterpret_cast<uintptr_t>(route) % 4) return MGEMV_ERR_ALIGNMENT;
   if (m_batch < 1 || m_batch > MGEMV_MAX_M_BATCH) return MGEMV_ERR_BATCH;
   if (const int st = check_problem(weights, scale, zero_add, n_out, k, group_size, quant_op, weight_bits)) return st;
   if (x == nullptr || y == nullptr) return MGEMV_ERR_NULL_POINTER;
@@ -705,6 +707,8 @@ int gemv_any(const void* weights, const uint16_t* x, const uint16_t* scale, cons
   g.tail.stride_scale = stride_scale;
   g.tail.stride_bias = stride_bias;
   g.tail.stride_y = stride_y;
+  g.tail.route = route;
+  g.tail.route_extent = route_extent;
   g.grid = dim3((unsigned)(g.plan.wgs_per_xcd * kNumXcd), 1, (unsigned)batch_count);
   g.block = dim3((unsigned)(kWave * g.plan.split_k), (unsigned)g.plan.tiles_per_wg, 1);
   g.stream = static_cast<hipStream_t>(stream);
@@ -812,6 +816,28 @@ int mgemv_gemv_batched_bf16(const void* weights, const uint16_t* x, const uint16
   return mgemv::gemv_any(weights, x, scale, zero_add, bias, y, batch_count, n_out, m_batch, k, group_size, quant_op,
                          weight_bits, stride_weights, stride_x, stride_scale, stride_bias, stride_y, stream,
                          mgemv::kActBf16);
+}
+
+int mgemv_gemv_routed(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+                      const uint16_t* bias, uint16_t* y, const int32_t* route, int route_extent, int batch_count,
+                      int n_out, int m_batch, int k, int group_size, int quant_op, int weight_bits,
+                      int64_t stride_weights, int64_t stride_x, int64_t stride_scale, int64_t stride_bias,
+                      int64_t stride_y, void* stream) {
+  if (route == nullptr) return MGEMV_ERR_NULL_POINTER;
+  return mgemv::gemv_any(weights, x, scale, zero_add, bias, y, batch_count, n_out, m_batch, k, group_size, quant_op,
+                         weight_bits, stride_weights, stride_x, stride_scale, stride_bias, stride_y, stream,
+                         mgemv::kActF16, 1.0f, 1.0f, mgemv::kProbeNone, nullptr, 0, false, route, route_extent);
+}
+
+int mgemv_gemv_routed_bf16(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,
+                           const uint16_t* bias, uint16_t* y, const int32_t* route, int route_extent, int batch_count,
+                           int n_out, int m_batch, int k, int group_size, int quant_op, int weight_bits,
+                           int64_t stride_weights, int64_t stride_x, int64_t stride_scale, int64_t stride_bias,
+                           int64_t stride_y, void* stream) {
+  if (route == nullptr) return MGEMV_ERR_NULL_POINTER;
+  return mgemv::gemv_any(weights, x, scale, zero_add, bias, y, batch_count, n_out, m_batch, k, group_size, quant_op,
+                         weight_bits, stride_weights, stride_x, stride_scale, stride_bias, stride_y, stream,
+                         mgemv::kActBf16, 1.0f, 1.0f, mgemv::kProbeNone, nullptr, 0, false, route, route_extent);
 }
 
 int mgemv_gemv_bf16(const void* weights, const uint16_t* x, const uint16_t* scale, const uint16_t* zero_add,

@@ -42,6 +42,8 @@ struct GemvTail {
   int seq_base;        // VALU kernel: tiles / sequences ...
   int seq_rem;         // ... and tiles % sequences (the first seq_rem sequences get one tile more)
   long long stride_weights, stride_x, stride_scale, stride_bias, stride_y;  // per batch problem
+  const int* route;    // routed launch: problem b takes weights, scales, zeros and bias of entry route[b] of the stack
+  int route_extent;    // entries in the stack: a problem routed outside [0, route_extent) is left alone
   unsigned long long* trace;  // timeline probe: kTimelineWordsPerWave words per wave, else unused
 };
 
@@ -62,7 +64,12 @@ struct Problem {
 };
 
 constexpr uint32_t pack_steps(int ksteps, int steps_per_wave) { return (uint32_t)ksteps | ((uint32_t)steps_per_wave << 16); }
-constexpr uint32_t pack_group(int group_size, int tiles_per_wg) { return (uint32_t)group_size | ((uint32_t)tiles_per_wg << 24); }
+// group size in bits 0-23, tiles per workgroup in bits 24-30, bit 31: the launch is routed (GemvTail::route)
+constexpr uint32_t kRoutedLaunch = 0x80000000u;
+constexpr uint32_t pack_group(int group_size, int tiles_per_wg, bool routed) {
+  return (uint32_t)group_size | ((uint32_t)tiles_per_wg << 24) | (routed ? kRoutedLaunch : 0u);
+}
+constexpr int tiles_per_wg_of(uint32_t packed_group) { return (int)((packed_group >> 24) & 0x7fu); }
 
 // ---------------------------------------------------------------------------------------------
 // Which part of the problem a wave works on.  Plain integer functions, compiled for the device

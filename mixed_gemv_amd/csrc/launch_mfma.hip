@@ -44,18 +44,24 @@ gemv_mfma_kernel(const uint8_t* weights, const half_t* x, const half_t* scale, c
   p.workgroups = workgroups;
   p.wgs_per_xcd = wgs_per_xcd;
   p.group_size = (int)(packed_group & 0xffffffu);
-  p.tiles_per_wg = (int)(packed_group >> 24);
+  p.tiles_per_wg = tiles_per_wg_of(packed_group);
   asm volatile("" ::"s"(weights), "s"(x), "s"(scale), "s"(zero_add), "s"(n_out), "s"(k), "s"(packed_steps),
                "s"(workgroups), "s"(wgs_per_xcd), "s"(packed_group), "s"(tail.bias), "s"(tail.y), "s"(tail.split_k),
                "s"(tail.m_batch), "s"(tail.num_groups), "s"(tail.flags), "s"(tail.stride_weights), "s"(tail.stride_x), "s"(tail.stride_scale),
                "s"(tail.stride_bias), "s"(tail.stride_y));
   const long long batch = blockIdx.z;
-  p.weights += batch * tail.stride_weights;
+  long long owner = batch;  // routed launch: whose weights, scales, zeros and bias the problem takes
+  if (packed_group & kRoutedLaunch) {
+    const int entry = tail.route[batch];
+    if ((unsigned)entry >= (unsigned)tail.route_extent) return;  // whole workgroup, before any barrier
+    owner = entry;
+  }
+  p.weights += owner * tail.stride_weights;
   p.x += batch * tail.stride_x;
-  p.scale += batch * tail.stride_scale;
-  p.zero_add += batch * tail.stride_scale;
+  p.scale += owner * tail.stride_scale;
+  p.zero_add += owner * tail.stride_scale;
   const bool has_bias = tail.bias != nullptr;
-  tail.bias += batch * tail.stride_bias;
+  tail.bias += owner * tail.stride_bias;
   tail.y += batch * tail.stride_y;
   const int m_batch = tail.m_batch;
 
@@ -229,16 +235,22 @@ gemv_mfma_lds_kernel(const uint8_t* weights, const half_t* x, const half_t* scal
   p.workgroups = workgroups;
   p.wgs_per_xcd = (workgroups + kNumXcd - 1) / kNumXcd;
   p.group_size = (int)(packed_group & 0xffffffu);
-  p.tiles_per_wg = (int)(packed_group >> 24);
+  p.tiles_per_wg = tiles_per_wg_of(packed_group);
   const long long batch = blockIdx.z;
-  if (batch != 0) {
-    p.weights += batch * tail.stride_weights;
+  long long owner = batch;  // routed launch: whose weights, scales, zeros and bias the problem takes
+  if ((blockIdx.z | (packed_group & kRoutedLaunch)) != 0) {
+    if ((packed_group & kRoutedLaunch) != 0) {
+      const int entry = tail.route[batch];
+      if ((unsigned)entry >= (unsigned)tail.route_extent) return;  // whole workgroup, before any barrier
+      owner = entry;
+    }
+    p.weights += owner * tail.stride_weights;
     p.x += batch * tail.stride_x;
-    p.scale += batch * tail.stride_scale;
-    p.zero_add += batch * tail.stride_scale;
+    p.scale += owner * tail.stride_scale;
+    p.zero_add += owner * tail.stride_scale;
   }
   const bool has_bias = tail.bias != nullptr;
-  tail.bias += batch * tail.stride_bias;
+  tail.bias += owner * tail.stride_bias;
   tail.y += batch * tail.stride_y;
   const int m_batch = tail.m_batch;
 
@@ -384,7 +396,7 @@ template <int BITS, int QOP, int GPR, int T>
 hipError_t launch_mfma_kernel_t(const GemvLaunch& g) {
   return launch(gemv_mfma_kernel<BITS, QOP, GPR, T>, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale,
                 g.zero_add, g.n_out, g.k, pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups,
-                g.plan.wgs_per_xcd, pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+                g.plan.wgs_per_xcd, pack_group(g.group_size, g.plan.tiles_per_wg, g.tail.route != nullptr), g.tail);
 }
 
 template <int BITS, int QOP, int GPR>
@@ -448,7 +460,7 @@ hipError_t launch_mfma_lds_kernel_r(const GemvLaunch& g) {
   }
   return launch(kernel, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale, g.zero_add, g.n_out, g.k,
                 pack_steps(num_ksteps(g.k, BITS), g.plan.steps_per_wave), g.plan.workgroups, g.tail.num_groups,
-                pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+                pack_group(g.group_size, g.plan.tiles_per_wg, g.tail.route != nullptr), g.tail);
 }
 
 template <int BITS, int QOP, int GPR, int ACT>

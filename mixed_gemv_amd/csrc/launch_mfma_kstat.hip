@@ -68,14 +68,20 @@ gemv_mfma_kstat_kernel(const uint8_t* weights, const half_t* x, const half_t* sc
   p.group_size = (int)(packed_group & 0xffffffu);
   p.tiles_per_wg = 1;
   const long long batch = blockIdx.z;
-  if (batch != 0) {
-    p.weights += batch * tail.stride_weights;
+  long long owner = batch;  // routed launch: whose weights, scales, zeros and bias the problem takes
+  if ((blockIdx.z | (packed_group & kRoutedLaunch)) != 0) {
+    if ((packed_group & kRoutedLaunch) != 0) {
+      const int entry = tail.route[batch];
+      if ((unsigned)entry >= (unsigned)tail.route_extent) return;  // whole workgroup, before any barrier
+      owner = entry;
+    }
+    p.weights += owner * tail.stride_weights;
     p.x += batch * tail.stride_x;
-    p.scale += batch * tail.stride_scale;
-    p.zero_add += batch * tail.stride_scale;
+    p.scale += owner * tail.stride_scale;
+    p.zero_add += owner * tail.stride_scale;
   }
   const bool has_bias = tail.bias != nullptr;
-  tail.bias += batch * tail.stride_bias;
+  tail.bias += owner * tail.stride_bias;
   tail.y += batch * tail.stride_y;
   const int m_batch = tail.m_batch;
 
@@ -322,7 +328,7 @@ hipError_t launch_mfma_kstat_kernel(const GemvLaunch& g) {
     }
   }
   return launch(kernel, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale, g.zero_add, g.n_out, g.k,
-                pack_steps(num_ksteps(g.k, BITS), 1), g.plan.workgroups, g.tail.num_groups, pack_group(g.group_size, 1),
+                pack_steps(num_ksteps(g.k, BITS), 1), g.plan.workgroups, g.tail.num_groups, pack_group(g.group_size, 1, g.tail.route != nullptr),
                 g.tail);
 }
 

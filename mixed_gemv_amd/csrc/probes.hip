@@ -54,7 +54,7 @@ hipError_t launch_gemv_probe_kind(const GemvLaunch& g) {
   const auto args = [&](auto kernel) {
     return launch(kernel, g.grid, g.block, g.lds, g.stream, g.weights, g.x, g.scale, g.zero_add, g.n_out, g.k,
                   pack_steps(num_ksteps(g.k, 4), g.plan.steps_per_wave), g.plan.workgroups, g.tail.num_groups,
-                  pack_group(g.group_size, g.plan.tiles_per_wg), g.tail);
+                  pack_group(g.group_size, g.plan.tiles_per_wg, g.tail.route != nullptr), g.tail);
   };
   return g.plan.tiles_in_sequence > 1
              ? args(gemv_dpp_kernel<4, MGEMV_FINEGRAINED_SCALE_AND_ZEROS, 1, 1, true, kActF16, PROBE>)

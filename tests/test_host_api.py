@@ -201,6 +201,12 @@ def test_gemv_argument_checks_return_codes_without_launching():
     assert gemv(x=ctypes.c_void_p(0x1002)) == 13
     assert lib.mgemv_gemv_batched(p, p, p, p, None, p, 0, 64, 1, 512, 128, 3, 4, 0, 0, 0, 0, 0, None) == 8
     assert lib.mgemv_dequantize(p, p, p, None, 64, 512, 128, 3, 4, None) == 1
+    # routed launch: the route is required, its stack extent positive, its address a multiple of 4
+    routed = lambda r, extent, fn=lib.mgemv_gemv_routed: fn(p, p, p, p, None, p, r, extent, 2, 64, 1, 512, 128, 3, 4,  # noqa: E731
+                                                            0, 0, 0, 0, 0, None)
+    assert routed(None, 4) == 1 and routed(None, 4, lib.mgemv_gemv_routed_bf16) == 1
+    assert routed(p, 0) == 8 and routed(p, -3, lib.mgemv_gemv_routed_bf16) == 8
+    assert routed(ctypes.c_void_p(0x1002), 4) == 13
     assert lib.mgemv_dequantize(p, p, p, p, 64, 512, 16, 2, 4, None) == 5
     # per-column mode ignores group_size entirely (mixed_gemv_test.cu:142-143): 16 would be rejected otherwise
     assert lib.mgemv_dequantize(p, p, None, None, 64, 512, 16, 1, 4, None) == 1
