@@ -142,6 +142,41 @@ def test_an_index_outside_the_stack_leaves_its_outputs_alone(gpu, forced_variant
     assert np.array_equal(got[3], stack.single(0, 3))
 
 
+def test_a_captured_launch_follows_the_route_it_finds_at_replay(gpu):
+    """The kernel reads the indices, so a HIP graph captured once serves every later routing decision: the
+    route is rewritten in place between replays (by device-side work, as a router would)."""
+    import torch
+    case = CASES[0]
+    _, n_out, k, bits, qop, g, m, _, element, _, _ = case
+    stack = Stack(case, gpu, 3)
+    routes = [[0, 1, 2], [4, 4, 3], [2, 0, 4], [1, 3, 0]]
+    route = torch.tensor(routes[0], dtype=torch.int32, device=gpu)
+    y = torch.full((3, m, n_out), NAN_PATTERN, dtype=torch.int16, device=gpu)
+
+    def launch():
+        mg.device_gemv_routed(stack.w, stack.x, stack.scale, stack.zero, stack.bias, y, route, ENTRIES, 3, n_out, m, k,
+                              g, stack.strides(), qop, bits, element=element)
+
+    launch()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            launch()
+    torch.cuda.current_stream().wait_stream(side)
+    for r in routes:
+        route.copy_(torch.tensor(r, dtype=torch.int32, device=gpu))
+        y.fill_(NAN_PATTERN)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.cpu().numpy().view(np.uint16)
+        for b, entry in enumerate(r):
+            assert np.array_equal(got[b], stack.single(entry, b)), (r, b)
+
+
 def test_identity_route_is_the_batched_launch(gpu):
     import torch
     case = CASES[0]
