@@ -68,3 +68,48 @@ def test_random_shape_parity(gpu, cfg):
     else:
         _, rel, _ = error_report(y, ref)
         assert np.isfinite(y.astype(np.float32)).all() and rel <= 2e-3, rel
+
+
+def _k_stationary_cases():
+    """The fp16 problems of the sweep above that fit the k-stationary matrix-core kernel (one wave per k step:
+    at most 16 k steps), each with a seeded cap on the workgroups, so that walks of every length, ragged last
+    tiles and ragged last k steps meet that kernel too, whatever the launch rules would have picked."""
+    rng = np.random.default_rng(977)
+    out = []
+    for cfg in CASES:
+        tag, n_out, k, bits, qop, group, m_batch, bias, element = cfg
+        ksteps = -(-k // (512 if bits == 4 else 256))
+        if element != "f16" or ksteps > 16:
+            continue
+        rows = m_batch if m_batch > 1 else int(rng.choice([2, 3, 7, 11, 16]))
+        if n_out * k * rows > 40_000_000:
+            rows = 2
+        cap = int(rng.choice([0, 0, 8, 16, 40, 104]))
+        out.append((f"{tag}_rows{rows}_cap{cap}", cfg, rows, cap))
+    return out
+
+
+KS_CASES = _k_stationary_cases()
+
+
+@pytest.mark.parametrize("case", KS_CASES, ids=[c[0] for c in KS_CASES])
+def test_random_shape_parity_on_the_k_stationary_kernel(gpu, case):
+    import mixed_gemv_amd as mg
+    _, (tag, n_out, k, bits, qop, group, _, bias, _), rows, cap = case
+    prob = Problem(tag + "_ks", n_out, k, bits, qop, group, m_batch=rows, bias=bias, x_dist="normal" if n_out % 8 else "uniform")
+    dev = DeviceProblem(prob, gpu)
+    mg.set_matrix_core_threshold(1)
+    mg.set_matrix_core_variant(mg.MATRIX_CORE_K_STATIONARY)
+    mg.set_launch_override(0, 0, 0, cap)
+    try:
+        plan = mg.query_launch(n_out, rows, k, bits, prob.group_size)
+        assert plan["matrix_core"] == 3, plan
+        cov = mg.plan_coverage(n_out, rows, k, bits, prob.group_size)
+        assert cov["tiles_miscovered"] == 0 and cov["bad_waves"] == 0, cov
+        y = dev.run()
+    finally:
+        mg.set_launch_override(0, 0, 0, 0)
+        mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
+        mg.set_matrix_core_threshold(0)
+    _, rel, _ = error_report(y, prob.oracle_gemv(threads=16))
+    assert np.isfinite(y.astype(np.float32)).all() and rel <= 2e-3, rel
