@@ -257,6 +257,78 @@ class Workload:
             bias=self.bias.cpu().numpy() if self.bias is not None else None)
 
 
+class RoutedWorkload:
+    """A decode step's expert GEMVs: one token, `top` of `experts` matrices of one shape (int4 group-128
+    scale+zero, fp16), chosen per launch by a device-side index array -- one mgemv_gemv_routed launch, or
+    `top` ordinary launches.  The stack is larger than the Infinity Cache and launch i takes experts
+    i*top .. i*top+top-1, so every launch reads weights that have long left the caches."""
+
+    def __init__(self, device, n_out=1408, k=2048, group=128, experts=256, top=8, seed=99):
+        import numpy as np
+        import torch
+        import mixed_gemv_amd as mg
+        self.mg, self.np = mg, np
+        self.n_out, self.k, self.group, self.experts, self.top = n_out, k, group, experts, top
+        self.bits, self.quant_op, self.m_batch, self.element = 4, 3, 1, "f16"
+        gen = torch.Generator(device="cpu").manual_seed(seed)
+        groups = k // group
+        self.one = mg.preprocessed_size((k, n_out), mg.QuantType.W4_A16)
+        self.raw = torch.randint(0, 256, (experts, n_out * k // 2), dtype=torch.uint8, generator=gen).numpy()
+        pre = mg.MixedGemvWeightPreprocessor.run(self.raw.reshape(-1), (experts, k, n_out), mg.LayoutType.kColumnMajor,
+                                                 mg.QuantType.W4_A16)
+        self.w = torch.from_numpy(pre).to(device)
+        self.s = (torch.rand((experts, groups, n_out), generator=gen) * 0.019 + 0.001).half().to(device)
+        self.z = (torch.rand((experts, groups, n_out), generator=gen) * 0.1 - 0.05).half().to(device)
+        self.x = (torch.rand((1, k), generator=gen) * 2 - 1).half().to(device)
+        self.y = torch.zeros((top, n_out), dtype=torch.half, device=device)
+        self.sets = experts // top            # distinct launches before the rotation repeats
+        self.host_routes = [[(i * top + j) % experts for j in range(top)] for i in range(self.sets)]
+        self.routes = [torch.tensor(r, dtype=torch.int32, device=device) for r in self.host_routes]
+        self.strides = (self.one, 0, groups * n_out, 0, n_out)
+        self.bytes = top * (algorithmic_bytes(n_out, k, 4, 3, group, 1, False) - k * 2) + k * 2
+        self.routed = True
+        self.description = (f"one token, {top} of {experts} experts of {n_out}x{k} (int4 group-{group} scale+zero), "
+                            f"stack of {experts * self.one >> 20} MiB")
+
+    def rotation(self):
+        return self.sets
+
+    def launch(self, i):
+        j = i % self.sets
+        if self.routed:
+            self.mg.device_gemv_routed(self.w, self.x, self.s, self.z, None, self.y, self.routes[j], self.experts,
+                                       self.top, self.n_out, 1, self.k, self.group, self.strides)
+        else:
+            for slot, e in enumerate(self.host_routes[j]):
+                self.mg.device_gemv(self.w[e * self.one:(e + 1) * self.one], self.x, self.s[e], self.z[e], None,
+                                    self.y[slot], 1, self.n_out, 1, self.k, self.group)
+
+    def parity(self, threads):
+        """Launch 0 both ways: the same bits; and its first and last problem against the oracle."""
+        import oracle as orc
+        import torch
+        np = self.np
+        got = {}
+        for routed in (True, False):
+            self.routed = routed
+            self.y.fill_(float("nan"))
+            self.launch(0)
+            torch.cuda.synchronize()
+            got[routed] = self.y.cpu().numpy().copy()
+        self.routed = True
+        worst = 0.0
+        for slot in (0, self.top - 1):
+            e = self.host_routes[0][slot]
+            ref = orc.gemv(self.raw[e], self.x.cpu().numpy(), self.s[e].cpu().numpy(), self.z[e].cpu().numpy(), None,
+                           self.n_out, 1, self.k, self.group, 3, 4, threads=threads).reshape(-1).astype(np.float64)
+            y = got[True][slot].astype(np.float64)
+            floor = max(float(np.sqrt(np.mean(ref * ref))) * 2.0 ** -7, 2.0 ** -24)
+            worst = max(worst, float((np.abs(y - ref) / np.maximum(np.abs(ref), floor)).max()))
+        same = bool(np.array_equal(got[True].view(np.uint16), got[False].view(np.uint16)))
+        return {"tolerance_rel": 2e-3, "max_rel_err": worst, "problems_checked_against_the_oracle": 2,
+                "routed_launch_equals_separate_launches_bit_for_bit": same, "ok": bool(same and worst <= 2e-3)}
+
+
 def cpu_model():
     try:
         with open("/proc/cpuinfo") as f:
@@ -672,8 +744,8 @@ def measure(wl, steps, warmup, use_graph):
 
 
 # what `--extra default` measures beside the headline: every benchmark configuration (c4 at each
-# activation row count), the vocabulary projection, batched launches and the bfloat16 entry points
-DEFAULT_EXTRA = "c1,c2,c3a,c3b,c4:m1,c4:m2,c4:m4,c4:m8,c4:m16,c5,c5:m4,c5:m16,vocab,nsx8,nsx16,ns:bf16,c5:bf16"
+# activation row count), the vocabulary projection, batched and routed launches and the bfloat16 entry points
+DEFAULT_EXTRA = "c1,c2,c3a,c3b,c4:m1,c4:m2,c4:m4,c4:m8,c4:m16,c5,c5:m4,c5:m16,vocab,nsx8,nsx16,routed,ns:bf16,c5:bf16"
 
 
 def main():
@@ -689,7 +761,8 @@ def main():
     ap.add_argument("--extra", default=DEFAULT_EXTRA,
                     help="comma list of further workloads reported under 'other_workloads' ('' = none); "
                          "'<name>x<B>' runs B problems per launch through the batched entry point, "
-                         "'<name>:bf16' the bfloat16 entry point, '<name>:m<M>' M activation rows")
+                         "'<name>:bf16' the bfloat16 entry point, '<name>:m<M>' M activation rows, 'routed' one token's "
+                         "8 of 256 experts in one routed launch (and in 8 launches)")
     ap.add_argument("--extra-steps", type=int, default=200, help="timed steps of each further workload")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and every oracle check")
     ap.add_argument("--no-warm-cache", action="store_true",
@@ -821,6 +894,22 @@ def main():
     others = {}
     built = {}   # (base, element) -> Workload, reused across activation row counts
     for name in [n for n in args.extra.split(",") if n and n != args.workload]:
+        if name == "routed":
+            built.clear()
+            torch.cuda.empty_cache()
+            rw = RoutedWorkload(device)
+            entry = {"workload": rw.description + ", one routed launch (mgemv_gemv_routed)"}
+            entry.update(measure(rw, args.extra_steps, max(20, args.warmup // 4), use_graph))
+            rw.routed = False
+            apart = measure(rw, args.extra_steps, max(20, args.warmup // 4), use_graph)
+            rw.routed = True
+            entry["separate_launches"] = {"launches_per_step": rw.top, "kernel_us_avg_events": apart["kernel_us_avg_events"],
+                                          "us_per_call": apart["us_per_call"]}
+            if not args.no_cpu:
+                entry["parity"] = rw.parity(threads)
+            others[name] = entry
+            del rw
+            continue
         # "<workload>[x<B>][:bf16][:m<M>]"
         base, *mods = name.split(":")
         base, _, batch = base.partition("x")
