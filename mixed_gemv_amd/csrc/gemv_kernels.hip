@@ -354,7 +354,8 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     auto walk = [&]() { return ceil_div(tiles, lp.workgroups); };
     const long long park_bytes = (long long)kKSlices * m_batch * kKStationaryParkSlots * 16;  // per tile of a walk
     while (lp.workgroups < tiles &&
-           ((long long)walk() * ksteps * kUnitBytes >= (1ll << 31) || walk() * park_bytes > kMaxKStationaryLds))
+           ((long long)(walk() + 2) * ksteps * kUnitBytes >= (1ll << 31) ||  // (the loop requests up to two tiles past the walk)
+            walk() * park_bytes > kMaxKStationaryLds))
       lp.workgroups = lp.workgroups * 2 < tiles ? lp.workgroups * 2 : tiles;
     lp.tiles_in_sequence = walk();
     lp.wgs_per_xcd = ceil_div(lp.workgroups, kNumXcd);
