@@ -130,6 +130,7 @@ struct PlanKnobs {
   bool wide_waves = false;  // the kernel is one of those compiled for at most 8 waves per workgroup
   int stages = 0;           // VALU kernel: 0 = built-in rule (2: the next unit in flight while one is computed), 1, 2
   int num_cus = kNumCus;    // compute units of the device the launch goes to (256 on an unpartitioned MI355X)
+  bool generic_groups = false;  // the group size does not divide the k step: one scale / zero lookup per block of a unit
 };
 
 // Tuned plans by problem: (n_out, k, weight bits, group size or 0 for any, m_batch) -> knobs.
@@ -301,6 +302,9 @@ inline int lds_staged_tiles_per_wg(int tiles, int staged_rows, int cus) {
 //     12 rows 15.34 / 14.87; 22016x4096, walks of 6, 13.68 / 13.98 still ahead); level or behind where the two fill
 //     it alike (8192x6144 16 rows 10.44 / 9.90; 14336x8192 18.1 / 17.0; 14336x4096 12 rows 10.18 / 10.16) or where
 //     the partial sums of a walk do not fit the LDS and the workgroups double (32768x8192 35.1 / 30.0).
+//   * group sizes that do not divide the k step (one scale / zero lookup per block: PlanKnobs::generic_groups) stay
+//     with the other kernels, the caller sees to that: 11008x3072 g96 at 4 rows 10.98 / 9.61; 14336x4608 g96 16.0 /
+//     13.95; 28672x8064 g96 36.45 / 33.08; 8192x6144 g192 12.34 / 10.83; 20480x5120 g160 19.9 / 19.9.
 inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int cus) {
   if (m_batch == 1 || ksteps < 4) return false;  // a single row stays on the VALU kernel, whatever was measured (above)
   const int walk = ceil_div(tiles, cus);
@@ -339,7 +343,8 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   const bool kstat_exists = ksteps <= kMaxWavesPerWorkgroup && !knobs.wide_waves;
   const bool kstat_asked = mc && knobs.matrix_core_variant == MGEMV_MATRIX_CORE_K_STATIONARY;
   const bool kstat_by_rule = knobs.matrix_core_variant == MGEMV_MATRIX_CORE_AUTO && knobs.matrix_core_min_batch == 0 &&
-                             ov_sk == 0 && ov_tw == 0 && ov_t == 0 && use_k_stationary(m_batch, tiles, ksteps, bits, cus);
+                             ov_sk == 0 && ov_tw == 0 && ov_t == 0 && !knobs.generic_groups &&
+                             use_k_stationary(m_batch, tiles, ksteps, bits, cus);
   if (kstat_exists && (kstat_asked || kstat_by_rule)) {
     LaunchPlan lp{};
     lp.matrix_core = true;
@@ -649,6 +654,8 @@ int device_info(int device, DeviceInfo& info) {
 PlanKnobs knobs_for_element(int n_out, int k, int bits, int group_size, int m_batch, int act, int num_cus = kNumCus) {
   PlanKnobs knobs = knobs_for(n_out, k, bits, group_size, m_batch, act, num_cus);
   knobs.num_cus = num_cus;
+  // (a group as long as k is the per-column mode, whose kernels look one scale up per row)
+  knobs.generic_groups = group_size > 0 && group_size != k && groups_per_run(group_size, bits) == 4;
   if (act == kActBf16) {
     // bf16: of the matrix-core kernels only the LDS-staged one (needs two tiles); the VALU kernel's
     // fp32 dequantiser wants the registers of 8-wave workgroups

@@ -523,6 +523,22 @@ def test_builtin_launch_rules_on_the_shapes_they_were_measured_on(shape, want):
     assert got["workgroups"] * per_workgroup >= tiles
 
 
+def test_group_sizes_that_do_not_divide_the_k_step_stay_off_the_k_stationary_rule():
+    """With one scale / zero lookup per block (groups of 96, 160, 192 ...) the k-stationary kernel measured 10-17 %
+    behind the LDS-staged one (11008x3072 g96 at 4 rows 10.98 against 9.61 us; 28672x8064 g96 36.5 against 33.1;
+    8192x6144 g192 12.3 against 10.8): the rule leaves such launches where they were; naming the kernel still works."""
+    for n_out, rows, k, group in [(11008, 4, 3072, 96), (28672, 2, 8064, 96), (8192, 4, 6144, 192), (20480, 3, 5120, 160)]:
+        assert mg.query_launch(n_out, rows, k, 4, 128 if k % 128 == 0 else 64)["matrix_core"] == 3, (n_out, k)
+        assert mg.query_launch(n_out, rows, k, 4, group)["matrix_core"] in (0, 2), (n_out, k, group)
+        mg.set_matrix_core_variant(mg.MATRIX_CORE_K_STATIONARY)
+        try:
+            assert mg.query_launch(n_out, rows, k, 4, group)["matrix_core"] == 3
+        finally:
+            mg.set_matrix_core_variant(mg.MATRIX_CORE_AUTO)
+    # per-column mode passes the reduction length as its group: regular
+    assert mg.query_launch(11008, 4, 4096, 4, 4096)["matrix_core"] == 3
+
+
 def test_bf16_launch_rules_differ_where_they_were_measured_to():
     """The bfloat16 kernels are bound by arithmetic: no tile walks, no whole-k single-wave workgroups,
     no two-unit waves; at most 8 waves per workgroup."""
