@@ -477,7 +477,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
   }
   int tiles_per_wg = pair_tiles ? 2 : 1;
   int workgroup_cap = 0;
-  if (!mc && tiles >= cus && ksteps >= 4) {
+  if (!mc && tiles >= cus && ksteps >= 5) {
     // "Exact fit": when the tiles divide (nearly) evenly over the compute units, one workgroup
     // of four waves per compute unit -- one wave per SIMD, all with the same amount of work --
     // beats any over-subscribed launch (8192x8192: 8.7 us against 10.2 us; 28672x8192: 2 %).
@@ -490,6 +490,12 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     for (int tw = 4; tw >= 1; tw /= 2) {
       const int sequences = cus * tw;
       if (ceil_div(tiles, sequences) > longest_walk) continue;
+      // The k steps must divide evenly over the 4 / tw waves of a sequence as well, or a SIMD of every compute
+      // unit idles (6 k steps on 4 waves are 2 + 2 + 2 + 0): against one workgroup per tile with a wave per k step,
+      // 12288x3072 7.09 us / 5.68, 20480x3072 10.10 / 8.79, 28672x3072 12.95 / 11.05, 12288x2560 7.13 / 5.24,
+      // 12288x3584 7.18 / 6.24, 12288x5120 9.39 / 8.58; with four k steps or fewer that launch is ahead on every
+      // even fit (12288x2048 5.10 / 4.52; 20480x2048 6.78 / 5.93; 28672x2048 8.32 / 7.64; 16384x2048 5.42 / 5.23).
+      if (ksteps % (4 / tw) != 0) continue;
       if ((long long)ceil_div(tiles, sequences) * sequences * 100 <= (long long)tiles * 103) {
         tiles_per_wg = tw;
         split_k = 4 / tw;

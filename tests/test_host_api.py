@@ -420,6 +420,13 @@ BUILTIN_PLANS = [
     ((28672, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256, split_k=4, tiles_in_sequence=7)),
     ((57344, 1, 8192), dict(matrix_core=0)),                   # a single row never goes to the matrix cores
     ((8192, 1, 8192), dict(matrix_core=0, workgroups=256, threads=256)),
+    # an even fit of the tiles is not enough for one four-wave workgroup per compute unit: the k steps must divide
+    # over its waves too, and there must be more than four of them
+    ((12288, 1, 3072), dict(matrix_core=0, workgroups=768, split_k=6, steps_per_wave=1, tiles_in_sequence=1)),
+    ((12288, 1, 2048), dict(matrix_core=0, workgroups=768, split_k=4, steps_per_wave=1, tiles_in_sequence=1)),
+    ((12288, 1, 5120), dict(matrix_core=0, workgroups=768, split_k=10, steps_per_wave=1, tiles_in_sequence=1)),
+    ((28672, 1, 5120), dict(matrix_core=0, workgroups=1792, split_k=1, steps_per_wave=10)),
+    ((12288, 1, 6144), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=3, tiles_in_sequence=3)),
     # at most one workgroup per compute unit: four k-split waves
     ((4096, 1, 4096), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=2)),
     ((4096, 1, 14336), dict(matrix_core=0, workgroups=256, split_k=4, steps_per_wave=7)),
