@@ -317,9 +317,23 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
     const long long park = (long long)walk * kKSlices * m_batch * kKStationaryParkSlots * 16;
     return bits == 4 && lds_slots16 * 10 >= slots * 11 && park <= kMaxKStationaryLds && (ksteps > 8 || walk <= 6);
   }
+  if (tiles <= cus) {
+    // At most one tile per compute unit, so no walk: still ahead of the VALU kernel's chunks of rows and of the
+    // LDS-staged kernel at 3-7 rows with 9-14 k steps (4096x4608 4 rows 5.38 / 6.53; 2048x5120 5.10 / 6.44; 3072x6144
+    // 5.43 / 6.29; 4096x6656 6.39 / 7.19; 3584x7168 6.31 / 7.14; 6 rows 4-7 % -- but 4096x7680, 15 k steps, 6 rows 7.72 /
+    // 6.92 and 4096x8192, 16 waves, 3 / 4 / 8 rows 7.44 / 6.70, 7.70 / 6.98, 8.38 / 7.21) and at 4-7 rows with 5-8
+    // (2560x2560 4 rows 4.35 / 4.74; 4096x3072 4.70 / 4.94; 4096x4096 6 rows 4.85 / 5.13; 3 rows lose 4-7 %; 8 rows
+    // level).  Measured from 128 tiles up, int4.
+    if (bits == 8 || tiles * 2 < cus || m_batch > 7) return false;
+    if (ksteps <= 8) return ksteps >= 5 && m_batch >= 4;
+    return m_batch >= 3 && (ksteps <= 14 || (ksteps == 15 && m_batch <= 4));
+  }
   if (bits == 8 && ksteps < 8) return false;  // 8192x1024 int8, 3 rows: 4.9 us against 4.6; 32768x1536: 10.9 / 10.3
   if (ksteps <= 8 || bits == 8) {
-    if (m_batch == 2) return ksteps == 8 && tiles * 2 >= cus * 5;  // the VALU kernel's two rows are cheap: 8192x4096 5.90 / 5.95
+    // the VALU kernel's two rows are cheap (8192x4096 5.90 / 5.95; 6144x3072 5.46 / 5.19; 12288x2560, 5 k steps, 6.71 /
+    // 5.57): from 6 k steps and 2.5 tiles per compute unit (10240x3584 7.01 / 7.27; 12288x3072 6.84 / 7.30; 18944x3584
+    // 9.88 / 10.47; 22016x3072 10.17 / 11.44; 37888x3584 15.89 / 17.87; 50304x3072 18.79 / 20.75)
+    if (m_batch == 2) return (bits == 8 ? ksteps == 8 : ksteps >= 6) && tiles * 2 >= cus * 5;
     return ksteps <= 5 ? tiles * 2 >= cus * 3 : tiles > cus;
   }
   const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);

@@ -559,9 +559,9 @@ FULL = [
 # Shapes that take the other branches of the launch heuristic (one four-wave workgroup per compute
 # unit with 4 / 2 / 1 tile sequences, with and without several tiles per sequence, with remainders).
 FIT = [
-    ("fit_tw4_two_tiles_each", 32032, 2048, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
+    ("fit_tw4_two_tiles_each", 32032, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
     ("fit_tw2_long_k", 8192, 28672, 4, SCALE_AND_ZEROS, 128, 1, True, "normal", (0.001, 0.02)),
-    ("fit_tw1_seven_tiles", 28672, 2048, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
+    ("fit_tw1_seven_tiles", 28672, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
     ("fit_int8_tw2", 8192, 4096, 8, PER_COLUMN, 0, 2, True, "uniform", (0.001, 0.01)),
 ]
 

@@ -451,8 +451,20 @@ BUILTIN_PLANS = [
     # ... and with a poor fit the k split stays
     ((17408, 1, 5120), dict(matrix_core=0, workgroups=1088, split_k=5, steps_per_wave=2)),
     # matrix cores: from 5 rows anywhere, from 3 rows on more than 256 tiles, from 2 rows on many tiles
-    ((4096, 4, 4096), dict(matrix_core=0)),
-    ((4096, 5, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
+    ((4096, 3, 4096), dict(matrix_core=0)),
+    ((4096, 4, 4096), dict(matrix_core=0, variant=mg.MATRIX_CORE_LDS_STAGED)),
+    ((4096, 5, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4, variant=mg.MATRIX_CORE_LDS_STAGED)),
+    # at most one tile per compute unit: the k-stationary kernel at 4-7 rows with 5-8 k steps, at 3-7 with 9-14
+    ((4096, 4, 4096), dict(matrix_core=3, workgroups=256, split_k=8, tiles_in_sequence=1)),
+    ((4096, 7, 4096), dict(matrix_core=3)),
+    ((2560, 4, 2560), dict(matrix_core=3, workgroups=160, split_k=5)),
+    ((2048, 3, 5120), dict(matrix_core=3, workgroups=128, split_k=10)),
+    ((4096, 6, 7168), dict(matrix_core=3)),
+    ((4096, 6, 7680), dict(matrix_core=2)),                    # 15 k steps: only up to 4 rows
+    ((4096, 4, 7680), dict(matrix_core=3)),
+    ((4096, 3, 8192), dict(matrix_core=0)),                    # 16 waves without a walk lose
+    ((4096, 4, 8192), dict(matrix_core=2)),
+    ((1024, 4, 6144), dict(matrix_core=0)),                    # fewer tiles than half the compute units: not measured
     ((16, 8, 4096), dict(matrix_core=1)),                      # a single tile: the register-operand kernel
     ((4096, 8, 4096), dict(matrix_core=2, tiles_per_wg=1, split_k=4)),
     ((5120, 3, 4096), dict(matrix_core=2, variant=mg.MATRIX_CORE_LDS_STAGED)),
