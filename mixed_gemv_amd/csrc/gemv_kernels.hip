@@ -401,6 +401,8 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;
     while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 8 * cus) split *= 2;
+    // three k steps: a wave each instead of 2 + 1 (2048x1408, 8 / 16 rows: 3.52 / 3.96 us against 4.11 / 4.69)
+    if (ksteps == 3 && split == 2 && max_split >= 3 && (long long)lp.workgroups * lp.tiles_per_wg * 3 <= 8 * cus) split = 3;
     // A split that leaves the last wave nearly idle (10 k steps over 4 waves: 3, 3, 3, 1) loses
     // to half as many evenly loaded waves, as long as the workgroup keeps four (5120x5120, 8 rows,
     // 2 tiles: 7.6 us at 2 waves per tile against 8.1 at 4; 6912x5120, 16 rows: 9.0 against 9.6;
