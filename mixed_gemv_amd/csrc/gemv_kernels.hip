@@ -315,7 +315,13 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
     const int tw16 = lds_staged_tiles_per_wg(tiles, 16, cus);
     const long long lds_slots16 = (long long)ceil_div(ceil_div(tiles, tw16), cus) * cus * tw16;
     const long long park = (long long)walk * kKSlices * m_batch * kKStationaryParkSlots * 16;
-    return bits == 4 && lds_slots16 * 10 >= slots * 11 && park <= kMaxKStationaryLds && (ksteps > 8 || walk <= 6);
+    // int8 weights: the operand is half as many registers and the stage half as long, and the kernel is ahead by
+    // 4-37 % on all 52 launches tried at 10-16 rows with 4-16 k steps and more tiles than compute units, as long as
+    // the partial sums of a walk fit the LDS (11008x4096 at 16 rows 10.74 us / 12.94; 18944x3584 14.80 / 19.09;
+    // 9216x3072 at 12 rows 7.80 / 10.67; 22016x2048 10.98 / 12.17; 11008x1024 5.78 / 6.14; where the workgroups double
+    // for the LDS it loses: 32000x4096 at 16 rows 25.66 / 24.19, 50304x2048 22.62 / 21.19)
+    if (bits == 8) return tiles > cus && park <= kMaxKStationaryLds;
+    return lds_slots16 * 10 >= slots * 11 && park <= kMaxKStationaryLds && (ksteps > 8 || walk <= 6);
   }
   if (tiles <= cus) {
     // At most one tile per compute unit, so no walk: still ahead of the VALU kernel's chunks of rows and of the

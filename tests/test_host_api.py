@@ -581,8 +581,14 @@ def test_int8_weights_keep_two_to_four_rows_on_the_valu_kernel():
     assert [q(4096, m, 11008) for m in (3, 4, 5)] == [0, 0, 2]
     assert [q(28672, m, 8192) for m in (2, 3, 4)] == [0, 2, 2]
     # ... unless the k-stationary kernel takes the launch: 8-16 k steps of 256, 3-8 rows, more tiles than compute units
-    assert [q(8192, m, 4096) for m in (2, 3, 4, 8, 9)] == [0, 3, 3, 3, 2]
+    assert [q(8192, m, 4096) for m in (2, 3, 4, 8)] == [0, 3, 3, 3]
     assert q(28672, 3, 4096) == 3 and q(28672, 2, 4096) == 0 and q(8192, 4, 1536) == 0 and q(4096, 8, 4096) == 2
+    # ... and at 9-16 rows wherever there are more tiles than compute units and the partial sums of a walk fit the LDS
+    assert [q(8192, m, 4096) for m in (9, 12, 16)] == [3, 3, 3]
+    assert q(11008, 16, 1024) == 3 and q(18944, 12, 3584) == 3
+    assert q(4096, 12, 4096) == 2                     # at most one tile per compute unit
+    assert q(32000, 16, 4096) == 2 and q(32000, 10, 4096) == 3 and q(50304, 16, 2048) == 2   # walks of 8 and 13 tiles
+    assert q(8192, 12, 8192) == 2                     # 32 k steps of 256: more than a workgroup has waves
 
 
 def test_default_plan_table_is_the_shipped_json_and_applies_to_256_compute_units_only():
