@@ -473,10 +473,14 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // One or two rows and up to 8 k steps: workgroups of up to 8 one-unit waves stay ahead of two-unit
     // waves well past 8192 waves (22016x4096, 11008 waves: 10.9 us against 11.8; 27200x4096,
     // 13600 waves: 12.6 against 13.0; 36864x2560: 11.8 against 12.3).
-    const bool short_single_row = !mc && m_batch <= 2 && ksteps <= 8;
+    // (int8 weights: the same reductions are twice as many k steps, and with half the arithmetic per byte more,
+    // shorter waves stay ahead there as well -- 22016x4096 at 1 / 2 rows 15.6 / 15.5 us with 8 waves per tile against
+    // 16.6 / 17.1 with 4; 11008x4096 at 2 rows 8.93 / 9.61; 12288x4096 9.55 / 10.19; 28672x4096 19.1 / 20.2.)
+    const bool short_single_row = !mc && m_batch <= 2 && ksteps <= (bits == 8 ? 16 : 8);
     const int kWaveBudget = (short_single_row ? 64 : 32) * cus;
     const int kSimds = cus * 4;
     split_k = ksteps < max_waves ? ksteps : max_waves;
+    if (short_single_row && bits == 8 && split_k > 8) split_k = 8;  // 16 one-unit waves lose: 11008x4096, 2 rows, 11.0 us / 8.9
     // One wave per unit does not fit the machine at once, and one wave per tile fills at least
     // 80 % of the SIMDs of its last round: the whole-k waves win (13824x5120: 9.1 us against
     // 10.3 at 5 waves per tile; 27648x5120: 15.6 against 17.5 at 3; 14848x6144: 10.6 against 12.1
@@ -492,7 +496,7 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // From 16 k steps four waves with longer pipelines are level with or ahead of more, shorter
     // ones (9216x14336: 16.9 us against 18.1 at 7 waves; 10240x11008: 14.8 against 15.3 at 11;
     // 10240x8192 and 11008x8192: level).
-    if (!mc && ksteps >= 16 && split_k > 4) split_k = 4;
+    if (!mc && !short_single_row && ksteps >= 16 && split_k > 4) split_k = 4;
     // The bfloat16 kernels are bound by their arithmetic, and two-unit waves are their worst
     // length by far (13824x5120: 18.9 us at 5 waves of 2 units against 14.0 at 2 waves of 5).
     if (knobs.wide_waves && !mc && split_k > 1 && ceil_div(ksteps, split_k) == 2) split_k = (split_k + 1) / 2;
