@@ -82,6 +82,14 @@ def lib():
             raise ImportError(
                 f"{LIB_PATH} not found: the HIP library is not built "
                 "(run `python -m mixed_gemv_amd.build`); there is no CPU fallback")
+        # PyTorch ships a HIP runtime of its own.  The library must bind to the runtime that owns the memory of the
+        # tensors it is handed, so that runtime has to be in the process before the library is loaded: loaded first,
+        # the library would bring in the system's runtime beside it, and every launch on a tensor would then fail
+        # with "no usable gfx950 device".
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         handle = ctypes.CDLL(LIB_PATH)
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(handle, name)

@@ -652,3 +652,15 @@ def test_an_entry_ships_only_after_two_confirmations():
     assert autotune.confirmed({"confirmations": [3.1, 0.4, 2.0]})
     assert not autotune.confirmed({"confirmations": [3.1, 2.4, -2.2]})      # behind once by as much as it gains
     assert autotune.confirmed({"confirmations": [5.0, 4.0]}, min_gain=0.04) and not autotune.confirmed({"confirmations": [5.0, 4.0]}, leases=3)
+
+
+def test_the_library_is_loaded_behind_pytorch():
+    """PyTorch brings its own HIP runtime; loaded in front of it, the library would bind to the system's runtime
+    instead and know nothing of the tensors' memory.  The loader therefore imports torch first."""
+    import subprocess
+    import sys
+    code = ("import sys, mixed_gemv_amd as mg; assert 'torch' not in sys.modules; mg.set_default_plans(True); "
+            "assert 'torch' in sys.modules; print('ok')")
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300,
+                         cwd=os.path.join(os.path.dirname(__file__), ".."))
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stderr[-2000:]
