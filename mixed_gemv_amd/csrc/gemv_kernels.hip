@@ -345,7 +345,9 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
   const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);
   const long long lds_slots = (long long)ceil_div(ceil_div(tiles, tw), cus) * cus * tw;
   if (lds_slots * 10 >= slots * 11) return m_batch >= 3 || walk >= 3;  // fills the machine better by a tenth or more
-  if (m_batch == 2) return walk == 3 || (walk > 3 && slots == tiles);
+  // two rows: from walks of 3 tiles, evenly filled or not (21024x7808, walks of 6 at 85 %, 19.1 us / 21.8; 22016x8192 20.1 /
+  // 22.2; 30064x6144 19.2 / 20.5; 14336x8192 and 16336x5632 level; 13824x5120, whose whole-k VALU waves fit well, 10.9 / 10.55)
+  if (m_batch == 2) return walk >= 3;
   if (m_batch <= 4) return walk == 2 || walk == 3 || slots == tiles;
   return walk == 2 && ksteps <= 12;
 }
@@ -401,12 +403,21 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     lp.matrix_core = true;
     lp.staged_rows = m_batch <= 8 ? 8 : 16;
     lp.tiles_per_wg = lds_staged_tiles_per_wg(tiles, lp.staged_rows, cus);
+    // Long reductions on many tiles (more than 16 k steps, more than 4 tiles per compute unit; the k-stationary kernel
+    // does not reach these) want about two workgroups per compute unit, of few waves that walk the whole reduction:
+    // 2 tiles per workgroup, or 4 where that still leaves more than 2.75 workgroups per compute unit; up to 8 rows,
+    // workgroups of 2 tiles split k in two.  Against what the rules above give (us): 34576x8576 at 12 rows 40.9 / 47.7;
+    // 33664x8832 at 16 rows 43.8 / 52.0; 19056x10112 at 3 / 12 rows 24.7 / 27.8, 32.8 / 38.1; 16400x9216 at 16 rows
+    // 29.4 / 35.0; 28672x8704 at 5 / 16 rows 29.0 / 32.2, 33.0 / 36.2; 22016x11008 at 8 rows 30.4 / 33.6.
+    const bool long_reduction = ksteps > 16 && tiles > 4 * cus;
+    if (long_reduction) lp.tiles_per_wg = ceil_div(tiles, 2) * 4 > cus * 11 ? 4 : 2;
     // the kernel exists for 2, 4, 8 or 16 staged rows per wave of a k range
     if (ov_tw > 0 && ov_tw <= 8 && lp.staged_rows % ov_tw == 0 && lp.staged_rows / ov_tw >= 2) lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
     const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;
     while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 8 * cus) split *= 2;
+    if (long_reduction) split = lp.staged_rows == 8 && lp.tiles_per_wg == 2 ? 2 : 1;
     // three k steps: a wave each instead of 2 + 1 (2048x1408, 8 / 16 rows: 3.52 / 3.96 us against 4.11 / 4.69)
     if (ksteps == 3 && split == 2 && max_split >= 3 && (long long)lp.workgroups * lp.tiles_per_wg * 3 <= 8 * cus) split = 3;
     // A split that leaves the last wave nearly idle (10 k steps over 4 waves: 3, 3, 3, 1) loses

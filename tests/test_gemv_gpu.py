@@ -590,7 +590,7 @@ def test_vocabulary_projection_one_tile_per_workgroup(gpu):
 # k split of the LDS-staged kernel.
 RULES = [
     ("whole_k_m1", 13824, 5120, 1, dict(matrix_core=0, threads=64, split_k=1, steps_per_wave=10)),
-    ("whole_k_m2", 13824, 5120, 2, dict(matrix_core=0, threads=64, split_k=1)),
+    ("whole_k_m2", 13824, 8704, 2, dict(matrix_core=0, threads=64, split_k=1)),   # (17 k steps: out of the k-stationary kernel's reach)
     ("one_unit_waves_m2", 6144, 4096, 2, dict(matrix_core=0, split_k=8, steps_per_wave=1)),
     ("one_unit_waves_11008_waves", 22016, 4096, 1, dict(matrix_core=0, split_k=8, workgroups=1376)),
     ("paired_tiles", 5120, 5120, 1, dict(matrix_core=0, tiles_per_wg=2, split_k=2, workgroups=160)),
@@ -605,6 +605,11 @@ RULES = [
     ("four_tiles_160_workgroups", 10240, 8192, 8, dict(matrix_core=2, tiles_per_wg=4, workgroups=160, variant="lds_staged")),
     ("k_stationary_better_filled", 10240, 8192, 8, dict(matrix_core=3, workgroups=256, tiles_in_sequence=3)),
     ("k_stationary_walks_of_2", 5120, 4096, 3, dict(matrix_core=3, workgroups=256, tiles_in_sequence=2)),
+    # long reductions on many tiles (17 k steps, 1025 / 1792 tiles): about two workgroups per compute unit
+    ("long_k_two_tiles_split_in_two", 16400, 8704, 5, dict(matrix_core=2, tiles_per_wg=2, split_k=2, workgroups=520)),
+    ("long_k_two_tiles_whole_k", 16400, 8704, 12, dict(matrix_core=2, tiles_per_wg=2, split_k=1, workgroups=520)),
+    ("long_k_four_tiles_of_two_rows_each", 28672, 8704, 3, dict(matrix_core=2, tiles_per_wg=4, split_k=1, workgroups=448)),
+    ("two_rows_on_uneven_walks", 21024, 7808, 2, dict(matrix_core=3, workgroups=256, tiles_in_sequence=6)),
 ]
 
 
