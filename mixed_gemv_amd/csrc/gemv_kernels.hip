@@ -321,6 +321,11 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
     // 9216x3072 at 12 rows 7.80 / 10.67; 22016x2048 10.98 / 12.17; 11008x1024 5.78 / 6.14; where the workgroups double
     // for the LDS it loses: 32000x4096 at 16 rows 25.66 / 24.19, 50304x2048 22.62 / 21.19)
     if (bits == 8) return tiles > cus && park <= kMaxKStationaryLds;
+    // a tile count that leaves the LDS-staged kernel only pairs of tiles on a large matrix: ahead even where the partial
+    // sums of a walk need twice the workgroups (36400x5376 at 12 / 16 rows 23.1 / 29.3 us against 33.5 / 35.0)
+    if (tw16 <= 2 && tiles > 4 * cus) return true;
+    // up to 12 rows on walks of 2: 5120x5120 7.86 / 8.89; 7792x6016 8.98 / 9.83; 6144x4096 6.95 / 7.32; 8192x8192 level
+    if (m_batch <= 12 && walk == 2 && park <= kMaxKStationaryLds) return true;
     return lds_slots16 * 10 >= slots * 11 && park <= kMaxKStationaryLds && (ksteps > 8 || walk <= 6);
   }
   if (tiles <= cus) {
@@ -344,10 +349,17 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
   }
   const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);
   const long long lds_slots = (long long)ceil_div(ceil_div(tiles, tw), cus) * cus * tw;
+  // tile counts that leave the LDS-staged kernel without a tidy grouping (it falls back to a workgroup per tile, no
+  // stage shared): 16880x5376 at 3 / 5 / 8 rows 12.6 / 12.9 / 14.0 us against 17.4 / 17.7 / 17.8; 17408x8192 17.2 / 17.6 /
+  // 18.4 against 24.1 / 24.1 / 24.3
+  if (tw == 1 && tiles > 2 * cus && m_batch >= 3) return true;
   if (lds_slots * 10 >= slots * 11) return m_batch >= 3 || walk >= 3;  // fills the machine better by a tenth or more
   // two rows: from walks of 3 tiles, evenly filled or not (21024x7808, walks of 6 at 85 %, 19.1 us / 21.8; 22016x8192 20.1 /
   // 22.2; 30064x6144 19.2 / 20.5; 14336x8192 and 16336x5632 level; 13824x5120, whose whole-k VALU waves fit well, 10.9 / 10.55)
   if (m_batch == 2) return walk >= 3;
+  // walks of 4 up to 5 rows and 15 k steps: 13584x5632 11.1-11.2 / 12.0; 15360x6144 11.6-11.7 / 12.4-12.5; 12480x7424
+  // 13.6-14.1 / 14.7; 16384x6144 at 5 rows 12.0 / 12.8 (13824x5120 10.9 / 10.7; with 16 k steps 13312x8192 15.1 / 14.7)
+  if (m_batch <= 5 && walk == 4 && ksteps <= 15) return true;
   if (m_batch <= 4) return walk == 2 || walk == 3 || slots == tiles;
   return walk == 2 && ksteps <= 12;
 }
@@ -416,7 +428,10 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
     const int max_split = kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg < 4 ? kMaxWavesPerMfmaWorkgroup / lp.tiles_per_wg : 4;
     int split = 1;
-    while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= 8 * cus) split *= 2;
+    // (a tile count that left every tile a workgroup of its own, on a large matrix: single-wave workgroups are the worst
+    // of all -- 16880x5376 bf16 at 5 rows 28.7 us against 22.6 with four k-split waves -- so those may use twice the waves)
+    const int lds_wave_budget = (lp.tiles_per_wg == 1 && tiles > 2 * cus ? 20 : 8) * cus;
+    while (split < max_split && split * 2 <= ksteps && (long long)lp.workgroups * lp.tiles_per_wg * split * 2 <= lds_wave_budget) split *= 2;
     if (long_reduction) split = lp.staged_rows == 8 && lp.tiles_per_wg == 2 ? 2 : 1;
     // three k steps: a wave each instead of 2 + 1 (2048x1408, 8 / 16 rows: 3.52 / 3.96 us against 4.11 / 4.69)
     if (ksteps == 3 && split == 2 && max_split >= 3 && (long long)lp.workgroups * lp.tiles_per_wg * 3 <= 8 * cus) split = 3;
