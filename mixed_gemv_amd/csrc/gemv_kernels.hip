@@ -345,6 +345,9 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
     // 5.57): from 6 k steps and 2.5 tiles per compute unit (10240x3584 7.01 / 7.27; 12288x3072 6.84 / 7.30; 18944x3584
     // 9.88 / 10.47; 22016x3072 10.17 / 11.44; 37888x3584 15.89 / 17.87; 50304x3072 18.79 / 20.75)
     if (m_batch == 2) return (bits == 8 ? ksteps == 8 : ksteps >= 6) && tiles * 2 >= cus * 5;
+    // five waves on four SIMDs: one SIMD carries two of them through every tile, and on longer walks the LDS-staged
+    // kernel is ahead (26208x2176 at 3 rows 10.1 us / 11.3; 30112x2176 10.3 / 12.1; 14240x2560 at 8 rows 7.3 / 7.8)
+    if (ksteps == 5 && walk >= 4) return false;
     return ksteps <= 5 ? tiles * 2 >= cus * 3 : tiles > cus;
   }
   const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);
@@ -361,7 +364,9 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
   // 13.6-14.1 / 14.7; 16384x6144 at 5 rows 12.0 / 12.8 (13824x5120 10.9 / 10.7; with 16 k steps 13312x8192 15.1 / 14.7)
   if (m_batch <= 5 && walk == 4 && ksteps <= 15) return true;
   if (m_batch <= 4) return walk == 2 || walk == 3 || slots == tiles;
-  return walk == 2 && ksteps <= 12;
+  // 5-8 rows: walks of 2 up to 12 k steps, and walks of 5 or more (22144x7936 at 6 rows 20.9 us / 23.8; 20672x8064 at 8
+  // rows 20.3 / 23.1; 23104x7680 at 5 rows 20.8 / 23.1; 29024x5760 19.3 / 21.2); walks of 4 lose 3-5 % at 6-8 rows
+  return (walk == 2 && ksteps <= 12) || walk >= 5;
 }
 
 LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs& knobs) {
@@ -548,6 +553,10 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
       // 12288x3584 7.18 / 6.24, 12288x5120 9.39 / 8.58; with four k steps or fewer that launch is ahead on every
       // even fit (12288x2048 5.10 / 4.52; 20480x2048 6.78 / 5.93; 28672x2048 8.32 / 7.64; 16384x2048 5.42 / 5.23).
       if (ksteps % (4 / tw) != 0) continue;
+      // ... and with up to 8 k steps a single tile sequence of four k-split waves (two units a wave, then the next
+      // tile) is behind a workgroup of one-unit waves per tile: 12288x4096 6.6 us / 7.3; 20480x4096 9.8 / 10.4; 20048x3840
+      // 10.0 / 11.0; 28672x4096 level (two or four sequences side by side stay: 16384x4096 8.0 / 9.0; 24576x3072 9.5 / 10.1)
+      if (ksteps <= 8 && tw == 1) continue;
       if ((long long)ceil_div(tiles, sequences) * sequences * 100 <= (long long)tiles * 103) {
         tiles_per_wg = tw;
         split_k = 4 / tw;

@@ -561,7 +561,7 @@ FULL = [
 FIT = [
     ("fit_tw4_two_tiles_each", 32032, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
     ("fit_tw2_long_k", 8192, 28672, 4, SCALE_AND_ZEROS, 128, 1, True, "normal", (0.001, 0.02)),
-    ("fit_tw1_seven_tiles", 28672, 4096, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
+    ("fit_tw1_seven_tiles", 28672, 6144, 4, SCALE_AND_ZEROS, 128, 1, False, "normal", (0.001, 0.02)),
     ("fit_int8_tw2", 8192, 4096, 8, PER_COLUMN, 0, 2, True, "uniform", (0.001, 0.01)),
 ]
 
