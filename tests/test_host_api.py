@@ -558,6 +558,22 @@ def test_group_sizes_that_do_not_divide_the_k_step_stay_off_the_k_stationary_rul
     assert mg.query_launch(11008, 4, 4096, 4, 4096)["matrix_core"] == 3
 
 
+def test_k_stationary_clauses_found_by_the_audits_of_random_shapes():
+    q = lambda n, m, k: mg.query_launch(n, m, k, 4, 128)["matrix_core"]  # noqa: E731
+    # tile counts that leave the LDS-staged kernel no grouping (1055 and 1088 tiles; 2275 at 16 staged rows)
+    assert [q(16880, m, 5376) for m in (3, 5, 8)] == [3, 3, 3] and [q(17408, m, 8192) for m in (3, 8)] == [3, 3]
+    assert q(36400, 16, 5376) == 3
+    # walks of 4: up to 5 rows and 15 k steps; walks of 5 and more: also at 6-8 rows
+    assert [q(13584, m, 5632) for m in (3, 5, 6, 8)] == [3, 3, 2, 2] and q(13312, 3, 8192) == 2
+    assert [q(22144, m, 7936) for m in (5, 6, 8)] == [3, 3, 3]
+    # two rows: walks of 3 and more with 9-16 k steps, 2.5 tiles per compute unit with 6-8
+    assert q(21024, 2, 7808) == 3 and q(8192, 2, 8192) == 0 and q(12288, 2, 3072) == 3 and q(12288, 2, 2560) == 0
+    # 9-12 rows on walks of 2
+    assert [q(5120, m, 5120) for m in (9, 12, 13, 16)] == [3, 3, 2, 2]
+    # five waves on four SIMDs: not on walks of 4 and more
+    assert q(26208, 3, 2176) == 2 and q(14240, 8, 2560) == 2 and q(6912, 3, 2432) == 3
+
+
 def test_bf16_launch_rules_differ_where_they_were_measured_to():
     """The bfloat16 kernels are bound by arithmetic: no tile walks, no whole-k single-wave workgroups,
     no two-unit waves; at most 8 waves per workgroup."""
