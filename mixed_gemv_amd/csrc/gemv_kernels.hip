@@ -339,7 +339,12 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
     if (ksteps <= 8) return ksteps >= 5 && m_batch >= 4;
     return m_batch >= 3 && (ksteps <= 14 || (ksteps == 15 && m_batch <= 4));
   }
-  if (bits == 8 && ksteps < 8) return false;  // 8192x1024 int8, 3 rows: 4.9 us against 4.6; 32768x1536: 10.9 / 10.3
+  // tile counts that leave the LDS-staged kernel without a tidy grouping (it falls back to a workgroup per tile, no
+  // stage shared): 16880x5376 at 3 / 5 / 8 rows 12.6 / 12.9 / 14.0 us against 17.4 / 17.7 / 17.8; 17408x8192 17.2 / 17.6 /
+  // 18.4 against 24.1 / 24.1 / 24.3; int8 17728x1792 at 6 rows 7.9 / 10.2
+  const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);
+  if (tw == 1 && tiles > 2 * cus && m_batch >= 3) return true;
+  if (bits == 8 && ksteps < 7) return false;  // 8192x1024 int8, 3 rows: 4.9 us against 4.6; 32768x1536: 10.9 / 10.3 (but 11264x1792, 7 k steps, 4 rows: 5.9 / 7.0)
   if (ksteps <= 8 || bits == 8) {
     // the VALU kernel's two rows are cheap (8192x4096 5.90 / 5.95; 6144x3072 5.46 / 5.19; 12288x2560, 5 k steps, 6.71 /
     // 5.57): from 6 k steps and 2.5 tiles per compute unit (10240x3584 7.01 / 7.27; 12288x3072 6.84 / 7.30; 18944x3584
@@ -350,12 +355,7 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
     if (ksteps == 5 && walk >= 4) return false;
     return ksteps <= 5 ? tiles * 2 >= cus * 3 : tiles > cus;
   }
-  const int tw = lds_staged_tiles_per_wg(tiles, 8, cus);
   const long long lds_slots = (long long)ceil_div(ceil_div(tiles, tw), cus) * cus * tw;
-  // tile counts that leave the LDS-staged kernel without a tidy grouping (it falls back to a workgroup per tile, no
-  // stage shared): 16880x5376 at 3 / 5 / 8 rows 12.6 / 12.9 / 14.0 us against 17.4 / 17.7 / 17.8; 17408x8192 17.2 / 17.6 /
-  // 18.4 against 24.1 / 24.1 / 24.3
-  if (tw == 1 && tiles > 2 * cus && m_batch >= 3) return true;
   if (lds_slots * 10 >= slots * 11) return m_batch >= 3 || walk >= 3;  // fills the machine better by a tenth or more
   // two rows: from walks of 3 tiles, evenly filled or not (21024x7808, walks of 6 at 85 %, 19.1 us / 21.8; 22016x8192 20.1 /
   // 22.2; 30064x6144 19.2 / 20.5; 14336x8192 and 16336x5632 level; 13824x5120, whose whole-k VALU waves fit well, 10.9 / 10.55)
@@ -427,7 +427,13 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     // 33664x8832 at 16 rows 43.8 / 52.0; 19056x10112 at 3 / 12 rows 24.7 / 27.8, 32.8 / 38.1; 16400x9216 at 16 rows
     // 29.4 / 35.0; 28672x8704 at 5 / 16 rows 29.0 / 32.2, 33.0 / 36.2; 22016x11008 at 8 rows 30.4 / 33.6.
     const bool long_reduction = ksteps > 16 && tiles > 4 * cus;
-    if (long_reduction) lp.tiles_per_wg = ceil_div(tiles, 2) * 4 > cus * 11 ? 4 : 2;
+    // (Up to 8 rows, 4 tiles only where their workgroups fill the last round to three quarters -- 28672x8704 and int8
+    // 27216x4224 do, 23648x11392 and int8 33616x4352 do not: 4-12 % either way.)
+    if (long_reduction) {
+      const int wgs4 = ceil_div(tiles, 4);
+      const bool four = lp.staged_rows == 16 ? ceil_div(tiles, 2) * 4 > cus * 11 : wgs4 * 4 >= ceil_div(wgs4, cus) * cus * 3;
+      lp.tiles_per_wg = four ? 4 : 2;
+    }
     // the kernel exists for 2, 4, 8 or 16 staged rows per wave of a k range
     if (ov_tw > 0 && ov_tw <= 8 && lp.staged_rows % ov_tw == 0 && lp.staged_rows / ov_tw >= 2) lp.tiles_per_wg = ov_tw;
     lp.workgroups = ceil_div(tiles, lp.tiles_per_wg);
