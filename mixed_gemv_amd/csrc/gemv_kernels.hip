@@ -232,11 +232,11 @@ inline bool use_matrix_cores(int m_batch, int tiles, int ksteps, int forced, boo
   // 4 rows: 10.4 against 11.5) except the largest (28672x8192, 3 rows: 41.4 against 39.7).
   if (bits == 8) return m_batch >= 5 || (m_batch >= 3 && tiles >= 6 * cus);
   const long long units = (long long)tiles * ksteps;
-  // 4 rows on 129-256 tiles: the barrier-free one-tile matrix-core launch is ahead from 16 k steps
+  // 4 rows on up to 256 tiles: the barrier-free one-tile matrix-core launch is ahead from 16 k steps
   // (4096x8192: 6.9 us against 7.4; 4096x14336: 9.7 against 10.7; 3584x18944: 12.3 against 13.8)
   // and level below (4096x4096: 5.07 against 5.00); 2 and 3 rows stay on the VALU kernel there.
   return m_batch >= 5 || (m_batch >= 3 && tiles > cus && units >= 8ll * cus) ||
-         (m_batch >= 4 && tiles > cus / 2 && ksteps >= 16) ||
+         (m_batch >= 4 && tiles >= 2 && ksteps >= 16) ||  // also on few tiles: 1536x8960 7.4 / 8.2; 1024x14336 9.0 / 10.2; 512x16384 9.9 / 10.9
          (m_batch >= 2 && !bf16 && tiles >= 6 * cus && (ksteps >= 8 || units > 64ll * cus));  // bf16, 28672x8192, 2 rows: 40.6 us against 37.8
 }
 
