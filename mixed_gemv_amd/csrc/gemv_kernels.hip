@@ -363,7 +363,10 @@ inline bool use_k_stationary(int m_batch, int tiles, int ksteps, int bits, int c
   // walks of 4 up to 5 rows and 15 k steps: 13584x5632 11.1-11.2 / 12.0; 15360x6144 11.6-11.7 / 12.4-12.5; 12480x7424
   // 13.6-14.1 / 14.7; 16384x6144 at 5 rows 12.0 / 12.8 (13824x5120 10.9 / 10.7; with 16 k steps 13312x8192 15.1 / 14.7)
   if (m_batch <= 5 && walk == 4 && ksteps <= 15) return true;
-  if (m_batch <= 4) return walk == 2 || walk == 3 || slots == tiles;
+  // ... and up to 8 rows with 9-11 k steps (12480x5632 at 6 rows 10.8 / 11.9; 13584x5632 at 8 rows 11.4 / 12.2; with 12-16
+  // k steps 6-8 rows lose 3-5 %: 15360x6144, 14336x8192)
+  if (walk == 4 && ksteps <= 11) return true;
+  if (m_batch <= 4) return walk == 2 || walk == 3 || walk >= 5 || slots == tiles;  // (walks of 5 and more: 22944x7680 at 4 rows 19.7 / 22.4)
   // 5-8 rows: walks of 2 up to 12 k steps, and walks of 5 or more (22144x7936 at 6 rows 20.9 us / 23.8; 20672x8064 at 8
   // rows 20.3 / 23.1; 23104x7680 at 5 rows 20.8 / 23.1; 29024x5760 19.3 / 21.2); walks of 4 lose 3-5 % at 6-8 rows
   return (walk == 2 && ksteps <= 12) || walk >= 5;

@@ -566,7 +566,9 @@ def test_k_stationary_clauses_found_by_the_audits_of_random_shapes():
     assert [q(16880, m, 5376) for m in (3, 5, 8)] == [3, 3, 3] and [q(17408, m, 8192) for m in (3, 8)] == [3, 3]
     assert q(36400, 16, 5376) == 3
     # walks of 4: up to 5 rows and 15 k steps; walks of 5 and more: also at 6-8 rows
-    assert [q(13584, m, 5632) for m in (3, 5, 6, 8)] == [3, 3, 2, 2] and q(13312, 3, 8192) == 2
+    assert [q(15360, m, 6144) for m in (3, 5, 6, 8)] == [3, 3, 2, 2] and q(13312, 3, 8192) == 2
+    assert [q(13584, m, 5632) for m in (3, 6, 8)] == [3, 3, 3]          # 11 k steps: up to 8 rows
+    assert q(22944, 4, 7680) == 3                                        # walks of 6 at 3-4 rows too
     assert [q(22144, m, 7936) for m in (5, 6, 8)] == [3, 3, 3]
     # two rows: walks of 3 and more with 9-16 k steps, 2.5 tiles per compute unit with 6-8
     assert q(21024, 2, 7808) == 3 and q(8192, 2, 8192) == 0 and q(12288, 2, 3072) == 3 and q(12288, 2, 2560) == 0
