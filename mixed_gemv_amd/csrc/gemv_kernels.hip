@@ -522,12 +522,12 @@ LaunchPlan plan_launch(int n_out, int k, int bits, int m_batch, const PlanKnobs&
     split_k = ksteps < max_waves ? ksteps : max_waves;
     if (short_single_row && bits == 8 && split_k > 8) split_k = 8;  // 16 one-unit waves lose: 11008x4096, 2 rows, 11.0 us / 8.9
     // One wave per unit does not fit the machine at once, and one wave per tile fills at least
-    // 80 % of the SIMDs of its last round: the whole-k waves win (13824x5120: 9.1 us against
+    // 75 % of the SIMDs of its last round: the whole-k waves win (13824x5120: 9.1 us against
     // 10.3 at 5 waves per tile; 27648x5120: 15.6 against 17.5 at 3; 14848x6144: 10.6 against 12.1
     // at 6; 13824x8192: 12.6 against 13.7 at 8).  With a worse fit they lose (17408x5120, 1088
     // tiles: 13.8 against 12.4), and the halving below stands.
     const bool whole_k_waves = !mc && !knobs.wide_waves && m_batch <= 2 && (long long)groups * split_k > kWaveBudget &&
-                               (long long)tiles * 100 >= (long long)ceil_div(tiles, kSimds) * kSimds * 80;
+                               (long long)tiles * 100 >= (long long)ceil_div(tiles, kSimds) * kSimds * 75;  // (12432x6144, 76 %: 10.2 us / 11.5)
     if (whole_k_waves) split_k = 1;
     while (split_k > 1 && (long long)groups * split_k > kWaveBudget) split_k = (split_k + 1) / 2;
     if (!mc && !short_single_row && split_k > 1 && ceil_div(ksteps, split_k) < 2 &&
